@@ -1,0 +1,153 @@
+/*
+ * C ABI of the MI355X decision-forest inference runtime.
+ *
+ * Every entry point in the first part keeps the name, argument list and
+ * meaning of the reference runtime it stands in for
+ * (src/runtime/tbruntime.h:10-48 and src/runtime/runtime.cpp in the reference
+ * checkout; the line given with each declaration is the definition it
+ * replaces).  Handles are pointers passed as intptr_t / void*, created by the
+ * Create / Construct functions and released by the matching Delete / Destroy.
+ * The reference aborts on errors; here a failing call returns 0 / does nothing
+ * and leaves a message for tbmi_last_error().  Not thread-safe (neither is the
+ * reference: process-wide singletons and flags).
+ *
+ * Buffers of the reference entry points are caller-owned HOST memory:
+ * inputs  = batchSize x rowSize float32, row-major, contiguous;
+ * results = batchSize float32 (int8 class ids for multiclass models).
+ *
+ * The tbmi_ entry points in the second part have no counterpart in the
+ * reference: device-resident inference, parity dumps, timing and tuning.
+ */
+#ifndef TBRUNTIME_AMD_H
+#define TBRUNTIME_AMD_H
+
+#include <stdbool.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TBAMD_EXPORT __attribute__((visibility("default")))
+
+/* ---- execution (runtime.cpp:58, :69, :94, :103, :112) ---- */
+TBAMD_EXPORT void RunInference(intptr_t inferenceRunner, void *inputs, void *results);
+TBAMD_EXPORT void RunInferenceOnMultipleBatches(intptr_t inferenceRunner, void *inputs, void *results,
+                                                int32_t numRows);
+TBAMD_EXPORT int32_t GetBatchSize(intptr_t inferenceRunner);
+TBAMD_EXPORT int32_t GetRowSize(intptr_t inferenceRunner);
+TBAMD_EXPORT void DeleteInferenceRunner(intptr_t inferenceRunner);
+
+/* ---- compiler options (runtime.cpp:123-174) ---- */
+TBAMD_EXPORT intptr_t CreateCompilerOptions(void);
+TBAMD_EXPORT void DeleteCompilerOptions(intptr_t options);
+TBAMD_EXPORT void Set_numberOfFeatures(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_batchSize(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_tileSize(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_thresholdTypeWidth(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_returnTypeWidth(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_returnTypeFloatType(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_featureIndexTypeWidth(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_nodeIndexTypeWidth(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_inputElementTypeWidth(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_tileShapeBitWidth(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_childIndexBitWidth(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_makeAllLeavesSameDepth(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_reorderTreesByDepth(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_statsProfileCSVPath(intptr_t options, const char *val);
+TBAMD_EXPORT void Set_pipelineSize(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_numberOfCores(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_numParallelTreeBatches(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_tilingType(intptr_t options, int32_t val); /* 0 uniform, 1 probabilistic, 2 hybrid */
+
+/* ---- GPU auto-schedule options (runtime.cpp:181-208) ---- */
+TBAMD_EXPORT intptr_t CreateGPUAutoScheduleOptions(void);
+TBAMD_EXPORT void DeleteGPUAutoScheduleOptions(intptr_t options);
+TBAMD_EXPORT void Set_numRowsPerTB(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_numRowsPerThread(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_rowTileSize(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_numTreeThreads(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_numTreesAtATime(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_cacheRows(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_cacheTrees(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_unrollTreeWalks(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_treeWalkInterleaveFactor(intptr_t options, int32_t val);
+TBAMD_EXPORT void Set_sharedMemoryReduce(intptr_t options, int32_t val);
+
+/* ---- compile (runtime.cpp:231, :283) ---- */
+TBAMD_EXPORT intptr_t CreateInferenceRunner(const char *modelJSONPath, const char *profileCSVPath,
+                                            intptr_t options);
+TBAMD_EXPORT intptr_t CreateInferenceRunnerForONNXModel(const char *modelPath, intptr_t options);
+
+/* ---- process-wide switches (runtime.cpp:301-325, :753) ---- */
+TBAMD_EXPORT void SetEnableSparseRepresentation(int32_t val);
+TBAMD_EXPORT int32_t IsSparseRepresentationEnabled(void);
+TBAMD_EXPORT void SetPeeledCodeGenForProbabilityBasedTiling(int32_t val);
+TBAMD_EXPORT int32_t IsPeeledCodeGenForProbabilityBasedTilingEnabled(void);
+TBAMD_EXPORT void SetEnableMeasureGpuKernelTime(bool val);
+TBAMD_EXPORT void SetNumberOfKernelRuns(int32_t val);
+TBAMD_EXPORT int64_t GetGPUKernelExecutionTime(intptr_t inferenceRunner); /* microseconds */
+
+/* ---- context API used by the GPU path (runtime.cpp:363-412, :468, :769) ---- */
+TBAMD_EXPORT intptr_t ConstructTreebeardContext(const char *modelPath, const char *modelGlobalsJSONPath,
+                                                intptr_t options);
+TBAMD_EXPORT intptr_t ConstructTreebeardContextFromGPUAutoscheduleOptions(const char *modelPath,
+                                                                          const char *modelGlobalsJSONPath,
+                                                                          intptr_t options,
+                                                                          intptr_t gpuScheduleOptions);
+TBAMD_EXPORT void DestroyTreebeardContext(intptr_t tbContext);
+TBAMD_EXPORT void SetForestCreatorType(intptr_t tbContext, const char *creatorType); /* "xgboost_json" | "onnx_file" */
+TBAMD_EXPORT void SetRepresentationAndSerializer(intptr_t tbContext, const char *repType);
+TBAMD_EXPORT void *ConstructGPUInferenceRunnerFromTBContext(void *tbContext);
+TBAMD_EXPORT void *ConstructInferenceRunnerFromHIR(void *tbContext);    /* runtime.cpp:442 */
+TBAMD_EXPORT void *ConstructGPUInferenceRunnerFromHIR(void *tbContext); /* runtime.cpp:455 */
+TBAMD_EXPORT void BuildHIRRepresentation(void *tbContext);              /* runtime.cpp:418; loads the model */
+TBAMD_EXPORT void *findBestGPUScheduleAndCompileModel(void *tbContext);
+
+/* ------------------------------------------------------------------------ */
+/* Additions without a counterpart in the reference.  Functions returning    */
+/* int32_t return 0 on success and -1 on failure (see tbmi_last_error).      */
+/* ------------------------------------------------------------------------ */
+TBAMD_EXPORT const char *tbmi_last_error(void);
+TBAMD_EXPORT int32_t tbmi_device_count(void);
+
+/* Inference on rows already resident in device memory (any row count). */
+TBAMD_EXPORT int32_t tbmi_run_device(intptr_t runner, const float *deviceInputs, void *deviceResults, int64_t rows);
+/* Multiclass: arg-max class ids (int8), per-class sums and softmax (float32 [rows][classes]); any may be null. */
+TBAMD_EXPORT int32_t tbmi_run_device_multiclass(intptr_t runner, const float *deviceInputs, int64_t rows,
+                                                int8_t *deviceClassIds, float *deviceMargins,
+                                                float *deviceProbabilities);
+/* Parity check: id (in the model file's numbering) of the leaf each row reaches in each tree,
+ * int32 [rows][numTrees] in device memory. */
+TBAMD_EXPORT int32_t tbmi_dump_leaf_ids(intptr_t runner, const float *deviceInputs, int32_t *deviceLeafIds,
+                                        int64_t rows);
+/* Average kernel durations (ms) over `runs` launches, measured with HIP events on the runner's stream. */
+TBAMD_EXPORT int32_t tbmi_time_kernels(intptr_t runner, const float *deviceInputs, void *deviceResults,
+                                       int64_t rows, int32_t runs, double *walkMs, double *finalizeMs);
+/* Timed search over launch plans on the given rows; keeps the fastest plan. */
+TBAMD_EXPORT int32_t tbmi_autotune(intptr_t runner, const float *deviceInputs, int64_t rows, double *bestMs);
+/* Pins a launch plan (values <= 0 keep the current one). */
+TBAMD_EXPORT int32_t tbmi_set_plan(intptr_t runner, int32_t rowsPerBlock, int32_t interleave, int32_t groupBytes,
+                                   int32_t treeSlices);
+TBAMD_EXPORT int32_t tbmi_describe_plan(intptr_t runner, char *buffer, int32_t length);
+TBAMD_EXPORT int32_t tbmi_num_trees(intptr_t runner);
+TBAMD_EXPORT int32_t tbmi_num_classes(intptr_t runner);
+
+/* Host-only model inspection (works without a GPU): loader and packer checks. */
+TBAMD_EXPORT intptr_t tbmi_load_forest(const char *modelPath, const char *creatorType, int32_t numberOfFeatures);
+TBAMD_EXPORT void tbmi_delete_forest(intptr_t forest);
+/* info[0..5] = numTrees, numFeatures, numClasses, transform, predicate, totalNodes; *initialValue */
+TBAMD_EXPORT int32_t tbmi_forest_info(intptr_t forest, int64_t *info, double *initialValue);
+TBAMD_EXPORT int32_t tbmi_forest_tree_size(intptr_t forest, int32_t tree);
+TBAMD_EXPORT int32_t tbmi_forest_tree(intptr_t forest, int32_t tree, float *value, int32_t *feature, int32_t *left,
+                                      int32_t *right, int32_t *classId);
+/* Packs the forest for the given plan and unpacks it again; returns the number of trees that differ
+ * from the (comparison-normalised) input, or -1 when the plan cannot hold the model.
+ * stats[0..4] = groups, bundles, nodes, ldsBytes, paddingTrees. */
+TBAMD_EXPORT int32_t tbmi_pack_roundtrip(intptr_t forest, int32_t rowsPerBlock, int32_t interleave,
+                                         int32_t groupBytes, int64_t *stats);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TBRUNTIME_AMD_H */

@@ -1,0 +1,54 @@
+// Device-facing model layout shared by the packer (host) and the HIP kernels.
+//
+// This replaces the reference's tiled-tree model buffers
+// (src/utils/TreeTilingUtils.cpp:363-413 tile byte layout, :434-495
+// offsets/lengths/classIds, src/mlir/Representations.cpp:1038-1052/:1728-1744
+// tile structs, src/gpu/GPURepresentations.cpp:90-256 device packing) with a
+// layout made for staging whole tree groups in LDS:
+//
+//  * A forest is cut into GROUPS of trees; one group's nodes are a contiguous
+//    run of 8-byte nodes that is copied verbatim into LDS, so every pointer a
+//    node holds is a byte address relative to the start of its group.
+//  * Node = { f32 value; u32 meta }.  value is the split threshold or, on a
+//    leaf, the prediction.  meta = (left-child byte address << 16) | feature
+//    offset.  The right child always follows the left one (+8 bytes).
+//  * The feature offset is pre-multiplied for the transposed row tile the
+//    kernel keeps in LDS (feature-major, one column per row of the block), so
+//    the address of the feature value is `featureOffset + 4*rowSlot`.
+//  * A leaf points at itself and tests the pad feature (index numFeatures),
+//    whose column holds -inf: `x < value` is then always true, the walk takes
+//    the "left" pointer and stays on the leaf.  A walk of `depth` steps thus
+//    needs no leaf test: it ends on the leaf for every row.
+//  * Trees are walked K at a time (a BUNDLE) to give every lane K independent
+//    dependency chains.  A bundle records the K root addresses, the trip count
+//    (deepest tree of the bundle) and the class the trees add to.
+#pragma once
+
+#include <cstdint>
+
+namespace tbamd {
+
+constexpr int kMaxInterleave = 8;
+constexpr uint32_t kNodeBytes = 8;
+
+struct DeviceNode {
+  float value;
+  uint32_t meta;
+};
+
+struct alignas(32) DeviceBundle {
+  uint16_t root[kMaxInterleave]; // byte address of each tree's root inside the group
+  uint16_t depth;                // walk steps that bring every row to a leaf
+  uint16_t classId;
+  uint32_t firstSlot;            // index of root[0] in the slot->tree table
+  uint32_t reserved[2];
+};
+
+struct DeviceGroup {
+  uint32_t nodeBegin;   // first node of the group in the packed node array
+  uint32_t nodeCount;   // multiple of 2 so that the group is a whole number of 16-byte pieces
+  uint32_t bundleBegin;
+  uint32_t bundleCount;
+};
+
+} // namespace tbamd

@@ -1,0 +1,56 @@
+// Host-callable launchers of the HIP kernels (kernels.hip).
+#pragma once
+
+#include "device_model.h"
+
+#include <hip/hip_runtime.h>
+
+namespace tbamd {
+
+// Scalars of the row-parallel walk (passed by value, live in SGPRs).
+struct WalkScalars {
+  int64_t rows = 0;
+  int32_t numFeatures = 0;
+  int32_t numClasses = 0;
+  int32_t numGroups = 0;
+  int32_t treeSlices = 1;
+  uint32_t groupRegionBytes = 0; // LDS bytes reserved for one tree group (multiple of 16)
+  int32_t transform = 0;         // 0 identity, 1 sigmoid
+  int32_t numTrees = 0;
+  double initialValue = 0.0;
+};
+
+struct WalkParams {
+  WalkScalars s;
+  const float *x = nullptr;       // rows x numFeatures, row-major, device
+  const uint4 *nodes16 = nullptr; // packed nodes viewed as 16-byte pieces
+  const DeviceBundle *bundles = nullptr;
+  const DeviceGroup *groups = nullptr;
+  float *out = nullptr;           // used when the epilogue is fused (1 slice, no classes)
+  double *partial = nullptr;      // [slices][rows][max(1, classes)] otherwise
+  // leaf-id dump (parity checks only)
+  int32_t *leafIds = nullptr;     // [rows][numTrees]
+  const int32_t *nodeOrigin = nullptr;
+  const int32_t *slotTree = nullptr;
+};
+
+struct FinalizeParams {
+  const double *partial = nullptr; // [slices][rows][max(1, classes)]
+  int64_t rows = 0;
+  int32_t numClasses = 0;
+  int32_t treeSlices = 1;
+  double initialValue = 0.0;
+  int32_t transform = 0;
+  float *out = nullptr;        // regression / binary prediction, may be null for multiclass
+  int8_t *classOut = nullptr;  // multiclass: arg-max class id
+  float *margins = nullptr;    // optional [rows][classes] per-class sums
+  float *probabilities = nullptr; // optional [rows][classes] softmax
+};
+
+// Row-parallel walk over LDS-staged tree groups.  `interleave` in {1,2,4,8};
+// `featureOffsetInWords` selects how node feature offsets are scaled.
+hipError_t LaunchWalkRowsLds(const WalkParams &p, int rowsPerBlock, int interleave, bool featureOffsetInWords,
+                             size_t ldsBytes, hipStream_t stream);
+hipError_t LaunchFinalize(const FinalizeParams &p, hipStream_t stream);
+
+} // namespace tbamd

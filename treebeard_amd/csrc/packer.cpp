@@ -1,0 +1,220 @@
+#include "packer.h"
+
+#include <algorithm>
+#include <cmath>
+#include <limits>
+#include <numeric>
+
+namespace tbamd {
+
+Forest NormalizeToLessThan(const Forest &forest) {
+  if (forest.predicate == Predicate::kLT) return forest;
+  Forest out = forest;
+  out.predicate = Predicate::kLT;
+  const bool swapChildren = forest.predicate == Predicate::kGE || forest.predicate == Predicate::kGT;
+  // x <= t  <=>  x < nextafter(t, +inf)   and   x > t  <=>  !(x <= t)
+  const bool bumpThreshold = forest.predicate == Predicate::kLE || forest.predicate == Predicate::kGT;
+  for (auto &tree : out.trees)
+    for (size_t i = 0; i < tree.NumNodes(); ++i) {
+      if (tree.IsLeaf((int32_t)i)) continue;
+      if (bumpThreshold) tree.value[i] = std::nextafter(tree.value[i], std::numeric_limits<float>::infinity());
+      if (swapChildren) std::swap(tree.left[i], tree.right[i]);
+    }
+  return out;
+}
+
+uint32_t PackedModel::PadFeatureOffset() const {
+  uint32_t words = (uint32_t)numFeatures * (uint32_t)plan.rowsPerBlock;
+  return plan.featureOffsetInWords ? words : words * 4u;
+}
+
+size_t PackedModel::LdsBytes() const {
+  return (size_t)(numFeatures + 1) * plan.rowsPerBlock * 4 + (size_t)maxGroupNodes * kNodeBytes;
+}
+
+namespace {
+
+// Level-order node list of one tree with siblings adjacent.
+struct LevelOrder {
+  std::vector<int32_t> order;    // packed position -> original node
+  std::vector<int32_t> position; // original node -> packed position
+};
+
+LevelOrder MakeLevelOrder(const Tree &tree) {
+  LevelOrder lo;
+  lo.position.assign(tree.NumNodes(), -1);
+  lo.order.push_back(0);
+  for (size_t head = 0; head < lo.order.size(); ++head) {
+    int32_t n = lo.order[head];
+    lo.position[n] = (int32_t)head;
+    if (tree.IsLeaf(n)) continue;
+    lo.order.push_back(tree.left[n]);
+    lo.order.push_back(tree.right[n]);
+  }
+  return lo;
+}
+
+} // namespace
+
+PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
+  const Forest forest = NormalizeToLessThan(input);
+  const int K = plan.interleave;
+  if (K < 1 || K > kMaxInterleave || (K & (K - 1))) throw Error("interleave must be 1, 2, 4 or 8");
+  if (plan.rowsPerBlock < 64 || (plan.rowsPerBlock & (plan.rowsPerBlock - 1)) || plan.rowsPerBlock > 1024)
+    throw Error("rowsPerBlock must be a power of two in [64, 1024]");
+  if (plan.groupBytes < 1024 || plan.groupBytes > 65536) throw Error("groupBytes must be in [1024, 65536]");
+
+  PackedModel pm;
+  pm.plan = plan;
+  pm.numFeatures = forest.numFeatures;
+  pm.numClasses = forest.numClasses;
+  pm.numTrees = (int32_t)forest.trees.size();
+  const uint64_t padOffset = pm.PadFeatureOffset();
+  if (padOffset > 0xFFFFu)
+    throw Error("feature offsets do not fit 16 bits for this rowsPerBlock / feature count");
+  const uint32_t featureStride = plan.featureOffsetInWords ? (uint32_t)plan.rowsPerBlock
+                                                           : (uint32_t)plan.rowsPerBlock * 4u;
+  const uint32_t groupCapacity = (uint32_t)plan.groupBytes / kNodeBytes;
+
+  // Order: class, then depth (the reference sorts by depth for its GPU schedules,
+  // src/mlir/GPUAutoSchedule.cpp:115-122); stable so equal keys keep model order.
+  std::vector<int32_t> depth(forest.trees.size());
+  for (size_t t = 0; t < forest.trees.size(); ++t) depth[t] = forest.trees[t].Depth();
+  std::vector<int32_t> order(forest.trees.size());
+  std::iota(order.begin(), order.end(), 0);
+  std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) {
+    int32_t ca = forest.numClasses > 0 ? forest.trees[a].classId : 0;
+    int32_t cb = forest.numClasses > 0 ? forest.trees[b].classId : 0;
+    if (ca != cb) return ca < cb;
+    return depth[a] < depth[b];
+  });
+
+  auto openGroup = [&]() {
+    DeviceGroup g{};
+    g.nodeBegin = (uint32_t)pm.nodes.size();
+    g.bundleBegin = (uint32_t)pm.bundles.size();
+    pm.groups.push_back(g);
+    // node 0 of every group: the null leaf padding trees point at
+    pm.nodes.push_back(DeviceNode{0.0f, (0u << 16) | (uint32_t)padOffset});
+    pm.nodeOrigin.push_back(-1);
+  };
+  auto closeGroup = [&]() {
+    DeviceGroup &g = pm.groups.back();
+    if ((pm.nodes.size() - g.nodeBegin) & 1) { // whole 16-byte pieces
+      pm.nodes.push_back(DeviceNode{0.0f, (0u << 16) | (uint32_t)padOffset});
+      pm.nodeOrigin.push_back(-1);
+    }
+    g.nodeCount = (uint32_t)pm.nodes.size() - g.nodeBegin;
+    g.bundleCount = (uint32_t)pm.bundles.size() - g.bundleBegin;
+    pm.maxGroupNodes = std::max(pm.maxGroupNodes, g.nodeCount);
+  };
+
+  size_t next = 0;
+  while (next < order.size()) {
+    openGroup();
+    DeviceGroup &g = pm.groups.back();
+    // one spare node keeps room for the alignment pad
+    auto freeNodes = [&]() { return groupCapacity - 1 - ((uint32_t)pm.nodes.size() - g.nodeBegin); };
+    bool any = false;
+    while (next < order.size()) {
+      // gather up to K consecutive trees of one class that still fit
+      DeviceBundle b{};
+      const int32_t cls = forest.numClasses > 0 ? forest.trees[order[next]].classId : 0;
+      uint32_t need = 0;
+      int count = 0;
+      while (count < K && next + count < order.size()) {
+        const Tree &tree = forest.trees[order[next + count]];
+        const int32_t c = forest.numClasses > 0 ? tree.classId : 0;
+        if (c != cls) break;
+        if ((uint32_t)tree.NumNodes() + 2 > groupCapacity)
+          throw Error("a tree of " + std::to_string(tree.NumNodes()) + " nodes does not fit one LDS tree group");
+        if (need + tree.NumNodes() > freeNodes()) break;
+        need += (uint32_t)tree.NumNodes();
+        ++count;
+      }
+      if (count == 0) break; // group full
+      b.classId = (uint16_t)cls;
+      b.firstSlot = (uint32_t)pm.slotTree.size();
+      for (int k = 0; k < K; ++k) {
+        if (k >= count) {
+          b.root[k] = 0; // null leaf
+          pm.slotTree.push_back(-1);
+          continue;
+        }
+        const int32_t t = order[next + k];
+        const Tree &tree = forest.trees[t];
+        const LevelOrder lo = MakeLevelOrder(tree);
+        const uint32_t base = (uint32_t)pm.nodes.size() - g.nodeBegin; // node index inside the group
+        b.root[k] = (uint16_t)(base * kNodeBytes);
+        b.depth = std::max<uint16_t>(b.depth, (uint16_t)depth[t]);
+        pm.slotTree.push_back(t);
+        for (size_t i = 0; i < lo.order.size(); ++i) {
+          const int32_t n = lo.order[i];
+          DeviceNode dn;
+          dn.value = tree.value[n];
+          if (tree.IsLeaf(n)) {
+            dn.meta = (((base + (uint32_t)i) * kNodeBytes) << 16) | (uint32_t)padOffset;
+          } else {
+            const uint32_t child = base + (uint32_t)lo.position[tree.left[n]];
+            if (lo.position[tree.right[n]] != lo.position[tree.left[n]] + 1)
+              throw Error("internal error: siblings not adjacent");
+            dn.meta = ((child * kNodeBytes) << 16) | ((uint32_t)tree.feature[n] * featureStride);
+          }
+          pm.nodes.push_back(dn);
+          pm.nodeOrigin.push_back(n);
+        }
+      }
+      pm.bundles.push_back(b);
+      next += count;
+      any = true;
+    }
+    closeGroup();
+    if (!any) throw Error("internal error: empty tree group");
+  }
+  if (pm.groups.empty()) { // a forest without trees still needs one (empty) group
+    openGroup();
+    closeGroup();
+  }
+  return pm;
+}
+
+Tree UnpackTree(const PackedModel &pm, int32_t treeIndex) {
+  const int K = pm.plan.interleave;
+  const uint32_t featureStride = pm.plan.featureOffsetInWords ? (uint32_t)pm.plan.rowsPerBlock
+                                                              : (uint32_t)pm.plan.rowsPerBlock * 4u;
+  for (const DeviceGroup &g : pm.groups)
+    for (uint32_t bi = g.bundleBegin; bi < g.bundleBegin + g.bundleCount; ++bi)
+      for (int k = 0; k < K; ++k) {
+        if (pm.slotTree[pm.bundles[bi].firstSlot + k] != treeIndex) continue;
+        // walk the packed tree breadth first, restoring original node ids
+        Tree tree;
+        tree.classId = pm.bundles[bi].classId;
+        std::vector<uint32_t> queue{pm.bundles[bi].root[k] / kNodeBytes};
+        size_t total = 0;
+        for (size_t head = 0; head < queue.size(); ++head) {
+          const DeviceNode &dn = pm.nodes[g.nodeBegin + queue[head]];
+          total = std::max<size_t>(total, (size_t)pm.nodeOrigin[g.nodeBegin + queue[head]] + 1);
+          const uint32_t child = (dn.meta >> 16) / kNodeBytes;
+          if (child != queue[head]) { queue.push_back(child); queue.push_back(child + 1); }
+        }
+        tree.value.assign(total, 0.f);
+        tree.feature.assign(total, 0);
+        tree.left.assign(total, -1);
+        tree.right.assign(total, -1);
+        for (uint32_t q : queue) {
+          const DeviceNode &dn = pm.nodes[g.nodeBegin + q];
+          const int32_t me = pm.nodeOrigin[g.nodeBegin + q];
+          const uint32_t child = (dn.meta >> 16) / kNodeBytes;
+          tree.value[me] = dn.value;
+          if (child != q) {
+            tree.feature[me] = (int32_t)((dn.meta & 0xFFFFu) / featureStride);
+            tree.left[me] = pm.nodeOrigin[g.nodeBegin + child];
+            tree.right[me] = pm.nodeOrigin[g.nodeBegin + child + 1];
+          }
+        }
+        return tree;
+      }
+  throw Error("tree not found in packed model");
+}
+
+} // namespace tbamd

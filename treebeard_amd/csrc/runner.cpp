@@ -1,0 +1,291 @@
+#include "runner.h"
+
+#include <algorithm>
+#include <sstream>
+
+namespace tbamd {
+
+bool gMeasureGpuKernelTime = false;
+int32_t gNumberOfKernelRuns = 1;
+
+namespace {
+
+void Check(hipError_t e, const char *what) {
+  if (e != hipSuccess) throw Error(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+template <typename T> T *Upload(const std::vector<T> &host, const char *what) {
+  T *ptr = nullptr;
+  const size_t bytes = std::max<size_t>(host.size(), 1) * sizeof(T);
+  Check(hipMalloc(reinterpret_cast<void **>(&ptr), bytes), what);
+  if (!host.empty()) Check(hipMemcpy(ptr, host.data(), host.size() * sizeof(T), hipMemcpyHostToDevice), what);
+  return ptr;
+}
+
+} // namespace
+
+InferenceRunner::InferenceRunner(Forest forest, const CompilerOptions &options,
+                                 const GPUAutoScheduleOptions *gpuOptions)
+    : m_forest(std::move(forest)), m_options(options) {
+  if (m_options.batchSize <= 0) throw Error("batchSize must be positive");
+  if (m_options.inputElementTypeWidth != 32) throw Error("only 32-bit float inputs are supported");
+  if (m_options.thresholdTypeWidth != 32) throw Error("only 32-bit float thresholds are supported");
+  if (m_forest.numClasses == 0 && (m_options.returnTypeWidth != 32 || !m_options.returnTypeFloatType))
+    throw Error("only 32-bit float predictions are supported");
+  m_forest.Validate();
+
+  int deviceCount = 0;
+  if (hipGetDeviceCount(&deviceCount) != hipSuccess || deviceCount == 0)
+    throw Error("no HIP device available: this library has no CPU fallback");
+  hipDeviceProp_t prop;
+  Check(hipGetDeviceProperties(&prop, 0), "hipGetDeviceProperties");
+  m_limits.computeUnits = prop.multiProcessorCount;
+  m_limits.ldsBytesPerBlock = (int32_t)std::min<size_t>(prop.sharedMemPerBlock, 160 * 1024);
+  Check(hipStreamCreateWithFlags(&m_stream, hipStreamNonBlocking), "hipStreamCreate");
+  Check(hipEventCreate(&m_evStart), "hipEventCreate");
+  Check(hipEventCreate(&m_evStop), "hipEventCreate");
+
+  m_model = PackForest(m_forest, ChoosePlan(m_forest, m_options.batchSize, gpuOptions, m_limits));
+  UploadModel();
+}
+
+InferenceRunner::~InferenceRunner() {
+  if (m_stream) (void)hipStreamSynchronize(m_stream);
+  FreeModel();
+  (void)hipFree(m_dPartial);
+  (void)hipFree(m_dStageIn);
+  (void)hipFree(m_dStageOut);
+  if (m_evStart) (void)hipEventDestroy(m_evStart);
+  if (m_evStop) (void)hipEventDestroy(m_evStop);
+  if (m_stream) (void)hipStreamDestroy(m_stream);
+}
+
+void InferenceRunner::FreeModel() {
+  (void)hipFree(m_dNodes);
+  (void)hipFree(m_dBundles);
+  (void)hipFree(m_dGroups);
+  (void)hipFree(m_dNodeOrigin);
+  (void)hipFree(m_dSlotTree);
+  m_dNodes = nullptr;
+  m_dBundles = nullptr;
+  m_dGroups = nullptr;
+  m_dNodeOrigin = nullptr;
+  m_dSlotTree = nullptr;
+}
+
+void InferenceRunner::UploadModel() {
+  // treeSlices never exceeds the number of groups the packer produced
+  m_model.plan.treeSlices = std::max(1, std::min<int32_t>(m_model.plan.treeSlices, (int32_t)m_model.groups.size()));
+  if (m_model.LdsBytes() > (size_t)m_limits.ldsBytesPerBlock) throw Error("launch plan exceeds the LDS of one workgroup");
+  m_dNodes = Upload(m_model.nodes, "upload nodes");
+  m_dBundles = Upload(m_model.bundles, "upload bundles");
+  m_dGroups = Upload(m_model.groups, "upload groups");
+  m_dNodeOrigin = Upload(m_model.nodeOrigin, "upload node origins");
+  m_dSlotTree = Upload(m_model.slotTree, "upload slot table");
+}
+
+void InferenceRunner::Repack(const LaunchPlan &plan) {
+  PackedModel next = PackForest(m_forest, plan);
+  Check(hipStreamSynchronize(m_stream), "hipStreamSynchronize");
+  FreeModel();
+  m_model = std::move(next);
+  UploadModel();
+}
+
+void InferenceRunner::EnsurePartial(int64_t rows) {
+  if (!NeedsFinalize()) return;
+  const size_t need = (size_t)m_model.plan.treeSlices * (size_t)rows * (size_t)std::max(1, m_forest.numClasses) * sizeof(double);
+  if (need <= m_partialBytes) return;
+  Check(hipStreamSynchronize(m_stream), "hipStreamSynchronize");
+  (void)hipFree(m_dPartial);
+  m_dPartial = nullptr;
+  m_partialBytes = 0;
+  Check(hipMalloc(reinterpret_cast<void **>(&m_dPartial), need), "allocate partial sums");
+  m_partialBytes = need;
+}
+
+void InferenceRunner::EnsureStaging() {
+  if (m_dStageIn) return;
+  const size_t rows = (size_t)m_options.batchSize;
+  Check(hipMalloc(reinterpret_cast<void **>(&m_dStageIn), rows * m_forest.numFeatures * sizeof(float)), "allocate input staging");
+  Check(hipMalloc(&m_dStageOut, rows * sizeof(float)), "allocate output staging");
+}
+
+WalkParams InferenceRunner::MakeWalkParams(const float *deviceInputs, int64_t rows) const {
+  WalkParams p;
+  p.s.rows = rows;
+  p.s.numFeatures = m_forest.numFeatures;
+  p.s.numClasses = m_forest.numClasses;
+  p.s.numGroups = (int32_t)m_model.groups.size();
+  p.s.treeSlices = m_model.plan.treeSlices;
+  p.s.groupRegionBytes = (uint32_t)m_model.maxGroupNodes * kNodeBytes;
+  p.s.transform = m_forest.transform == Transform::kSigmoid ? 1 : 0;
+  p.s.numTrees = (int32_t)m_forest.trees.size();
+  p.s.initialValue = m_forest.initialValue;
+  p.x = deviceInputs;
+  p.nodes16 = reinterpret_cast<const uint4 *>(m_dNodes);
+  p.bundles = m_dBundles;
+  p.groups = m_dGroups;
+  return p;
+}
+
+void InferenceRunner::Launch(const float *deviceInputs, int64_t rows, float *out, int8_t *classOut, float *margins,
+                             float *probabilities, int32_t *leafIds) {
+  if (rows <= 0) return;
+  EnsurePartial(rows);
+  WalkParams p = MakeWalkParams(deviceInputs, rows);
+  const bool finalize = NeedsFinalize();
+  p.out = finalize ? nullptr : out;
+  p.partial = finalize ? m_dPartial : nullptr;
+  if (leafIds) {
+    p.leafIds = leafIds;
+    p.nodeOrigin = m_dNodeOrigin;
+    p.slotTree = m_dSlotTree;
+  }
+  Check(LaunchWalkRowsLds(p, m_model.plan.rowsPerBlock, m_model.plan.interleave, m_model.plan.featureOffsetInWords,
+                          m_model.LdsBytes(), m_stream),
+        "launch walk kernel");
+  if (finalize) {
+    FinalizeParams f;
+    f.partial = m_dPartial;
+    f.rows = rows;
+    f.numClasses = m_forest.numClasses;
+    f.treeSlices = m_model.plan.treeSlices;
+    f.initialValue = m_forest.initialValue;
+    f.transform = p.s.transform;
+    f.out = out;
+    f.classOut = classOut;
+    f.margins = margins;
+    f.probabilities = probabilities;
+    Check(LaunchFinalize(f, m_stream), "launch finalize kernel");
+  }
+}
+
+void InferenceRunner::RunDevice(const float *deviceInputs, void *deviceResults, int64_t rows) {
+  const int runs = gMeasureGpuKernelTime ? std::max(1, gNumberOfKernelRuns) : 1;
+  if (gMeasureGpuKernelTime) Check(hipEventRecord(m_evStart, m_stream), "hipEventRecord");
+  for (int i = 0; i < runs; ++i) {
+    if (m_forest.numClasses > 0)
+      Launch(deviceInputs, rows, nullptr, static_cast<int8_t *>(deviceResults), nullptr, nullptr, nullptr);
+    else
+      Launch(deviceInputs, rows, static_cast<float *>(deviceResults), nullptr, nullptr, nullptr, nullptr);
+  }
+  if (gMeasureGpuKernelTime) Check(hipEventRecord(m_evStop, m_stream), "hipEventRecord");
+  Check(hipStreamSynchronize(m_stream), "inference kernels");
+  if (gMeasureGpuKernelTime) {
+    float ms = 0.f;
+    Check(hipEventElapsedTime(&ms, m_evStart, m_evStop), "hipEventElapsedTime");
+    m_lastKernelMicros = (int64_t)(ms * 1000.0);
+  }
+}
+
+void InferenceRunner::RunDeviceMulticlass(const float *deviceInputs, int64_t rows, int8_t *classIds, float *margins,
+                                          float *probabilities) {
+  if (m_forest.numClasses == 0) throw Error("model is not a multiclass classifier");
+  Launch(deviceInputs, rows, nullptr, classIds, margins, probabilities, nullptr);
+  Check(hipStreamSynchronize(m_stream), "inference kernels");
+}
+
+void InferenceRunner::DumpLeafIds(const float *deviceInputs, int32_t *deviceLeafIds, int64_t rows) {
+  // results of the prediction itself are discarded into the staging buffers
+  EnsurePartial(rows);
+  float *scratch = nullptr;
+  Check(hipMalloc(reinterpret_cast<void **>(&scratch), std::max<int64_t>(rows, 1) * sizeof(float)), "allocate scratch");
+  try {
+    Launch(deviceInputs, rows, scratch, reinterpret_cast<int8_t *>(scratch), nullptr, nullptr, deviceLeafIds);
+    Check(hipStreamSynchronize(m_stream), "leaf-id kernels");
+  } catch (...) {
+    (void)hipFree(scratch);
+    throw;
+  }
+  (void)hipFree(scratch);
+}
+
+void InferenceRunner::RunInference(const void *hostInputs, void *hostResults) {
+  EnsureStaging();
+  const size_t rows = (size_t)m_options.batchSize;
+  Check(hipMemcpyAsync(m_dStageIn, hostInputs, rows * m_forest.numFeatures * sizeof(float), hipMemcpyHostToDevice, m_stream), "copy inputs");
+  RunDevice(m_dStageIn, m_dStageOut, (int64_t)rows);
+  Check(hipMemcpy(hostResults, m_dStageOut, rows * ReturnTypeBytes(), hipMemcpyDeviceToHost), "copy results");
+}
+
+void InferenceRunner::TimeKernels(const float *deviceInputs, void *deviceResults, int64_t rows, int32_t runs,
+                                  double *walkMs, double *finalizeMs) {
+  runs = std::max(1, runs);
+  EnsurePartial(rows);
+  const bool finalize = NeedsFinalize();
+  WalkParams p = MakeWalkParams(deviceInputs, rows);
+  p.out = finalize ? nullptr : static_cast<float *>(deviceResults);
+  p.partial = finalize ? m_dPartial : nullptr;
+  Check(hipEventRecord(m_evStart, m_stream), "hipEventRecord");
+  for (int i = 0; i < runs; ++i)
+    Check(LaunchWalkRowsLds(p, m_model.plan.rowsPerBlock, m_model.plan.interleave, m_model.plan.featureOffsetInWords,
+                            m_model.LdsBytes(), m_stream),
+          "launch walk kernel");
+  Check(hipEventRecord(m_evStop, m_stream), "hipEventRecord");
+  Check(hipStreamSynchronize(m_stream), "walk kernel");
+  float ms = 0.f;
+  Check(hipEventElapsedTime(&ms, m_evStart, m_evStop), "hipEventElapsedTime");
+  if (walkMs) *walkMs = ms / runs;
+  if (finalizeMs) *finalizeMs = 0.0;
+  if (finalize) {
+    FinalizeParams f;
+    f.partial = m_dPartial;
+    f.rows = rows;
+    f.numClasses = m_forest.numClasses;
+    f.treeSlices = m_model.plan.treeSlices;
+    f.initialValue = m_forest.initialValue;
+    f.transform = p.s.transform;
+    if (m_forest.numClasses > 0) f.classOut = static_cast<int8_t *>(deviceResults);
+    else f.out = static_cast<float *>(deviceResults);
+    Check(hipEventRecord(m_evStart, m_stream), "hipEventRecord");
+    for (int i = 0; i < runs; ++i) Check(LaunchFinalize(f, m_stream), "launch finalize kernel");
+    Check(hipEventRecord(m_evStop, m_stream), "hipEventRecord");
+    Check(hipStreamSynchronize(m_stream), "finalize kernel");
+    Check(hipEventElapsedTime(&ms, m_evStart, m_evStop), "hipEventElapsedTime");
+    if (finalizeMs) *finalizeMs = ms / runs;
+  }
+}
+
+double InferenceRunner::AutoTune(const float *deviceInputs, int64_t rows) {
+  void *out = nullptr;
+  Check(hipMalloc(&out, std::max<int64_t>(rows, 1) * sizeof(float)), "allocate tuning output");
+  const LaunchPlan original = m_model.plan;
+  LaunchPlan best = original;
+  double bestMs = 1e300;
+  try {
+    for (const LaunchPlan &cand : CandidatePlans(m_forest, rows, m_limits)) {
+      try {
+        Repack(cand);
+      } catch (const Error &) {
+        continue; // plan cannot hold this model
+      }
+      double w = 0, f = 0;
+      TimeKernels(deviceInputs, out, rows, 1, &w, &f); // warm-up
+      TimeKernels(deviceInputs, out, rows, 3, &w, &f);
+      if (w + f < bestMs) {
+        bestMs = w + f;
+        best = m_model.plan;
+      }
+    }
+    Repack(best);
+  } catch (...) {
+    (void)hipFree(out);
+    throw;
+  }
+  (void)hipFree(out);
+  return bestMs;
+}
+
+std::string InferenceRunner::DescribePlan() const {
+  std::ostringstream os;
+  const LaunchPlan &p = m_model.plan;
+  os << "kernel=rows_lds rowsPerBlock=" << p.rowsPerBlock << " interleave=" << p.interleave
+     << " groupBytes=" << p.groupBytes << " treeSlices=" << p.treeSlices
+     << " offsetsInWords=" << (p.featureOffsetInWords ? 1 : 0) << " groups=" << m_model.groups.size()
+     << " bundles=" << m_model.bundles.size() << " nodes=" << m_model.nodes.size()
+     << " ldsBytes=" << m_model.LdsBytes();
+  return os.str();
+}
+
+} // namespace tbamd

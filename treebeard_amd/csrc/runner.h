@@ -1,0 +1,93 @@
+// Compiled model + device buffers + the RunInference entry points.
+//
+// Stands where the reference has InferenceRunnerBase / GPUInferenceRunner
+// (src/mlir/ExecutionHelpers.h:42-111, src/gpu/GPUExecutionHelper.h:34-60) and
+// the generated Prediction_Function's per-call alloc + H2D + kernel + D2H
+// (src/gpu/GPUSupportUtils.cpp:150-343).  Here the staging buffers are
+// allocated once per runner.
+#pragma once
+
+#include "forest.h"
+#include "kernels.h"
+#include "options.h"
+#include "packer.h"
+#include "tuner.h"
+
+#include <hip/hip_runtime.h>
+
+#include <string>
+
+namespace tbamd {
+
+// Process-wide switches of the reference's kernel-time shim
+// (src/gpu/GPUSupportUtils.cpp:52-104, :389-390).
+extern bool gMeasureGpuKernelTime;
+extern int32_t gNumberOfKernelRuns;
+
+class InferenceRunner {
+public:
+  InferenceRunner(Forest forest, const CompilerOptions &options, const GPUAutoScheduleOptions *gpuOptions);
+  ~InferenceRunner();
+  InferenceRunner(const InferenceRunner &) = delete;
+  InferenceRunner &operator=(const InferenceRunner &) = delete;
+
+  // Host buffers, exactly batchSize rows (src/runtime/runtime.cpp:58-67).
+  void RunInference(const void *hostInputs, void *hostResults);
+  // Device-resident rows; `out` is f32[rows] (int8[rows] for multiclass models).
+  void RunDevice(const float *deviceInputs, void *deviceResults, int64_t rows);
+  // Multiclass extras: any of the outputs may be null.
+  void RunDeviceMulticlass(const float *deviceInputs, int64_t rows, int8_t *classIds, float *margins,
+                           float *probabilities);
+  // Parity check: original leaf node id reached by every (row, tree), int32[rows][numTrees].
+  void DumpLeafIds(const float *deviceInputs, int32_t *deviceLeafIds, int64_t rows);
+  // Average duration in milliseconds of the walk kernel (and of the finalize
+  // kernel when the plan needs one) over `runs` launches, HIP events on the
+  // runner's stream.
+  void TimeKernels(const float *deviceInputs, void *deviceResults, int64_t rows, int32_t runs, double *walkMs,
+                   double *finalizeMs);
+  // Re-packs the model for another launch plan (used by the timed search).
+  void Repack(const LaunchPlan &plan);
+  // Timed search over CandidatePlans(); keeps the fastest.  Returns its time in ms.
+  double AutoTune(const float *deviceInputs, int64_t rows);
+
+  int32_t BatchSize() const { return m_options.batchSize; }
+  int32_t RowSize() const { return m_forest.numFeatures; }
+  int32_t NumTrees() const { return (int32_t)m_forest.trees.size(); }
+  int32_t NumClasses() const { return m_forest.numClasses; }
+  int32_t ReturnTypeBytes() const { return m_forest.numClasses > 0 ? 1 : 4; }
+  int64_t LastKernelMicros() const { return m_lastKernelMicros; }
+  const PackedModel &Model() const { return m_model; }
+  const Forest &GetForest() const { return m_forest; }
+  std::string DescribePlan() const;
+  hipStream_t Stream() const { return m_stream; }
+
+private:
+  void UploadModel();
+  void FreeModel();
+  void EnsurePartial(int64_t rows);
+  void EnsureStaging();
+  bool NeedsFinalize() const { return m_model.plan.treeSlices > 1 || m_forest.numClasses > 0; }
+  WalkParams MakeWalkParams(const float *deviceInputs, int64_t rows) const;
+  void Launch(const float *deviceInputs, int64_t rows, float *out, int8_t *classOut, float *margins,
+              float *probabilities, int32_t *leafIds);
+
+  Forest m_forest;
+  CompilerOptions m_options;
+  DeviceLimits m_limits;
+  PackedModel m_model;
+  hipStream_t m_stream = nullptr;
+  hipEvent_t m_evStart = nullptr, m_evStop = nullptr;
+
+  DeviceNode *m_dNodes = nullptr;
+  DeviceBundle *m_dBundles = nullptr;
+  DeviceGroup *m_dGroups = nullptr;
+  int32_t *m_dNodeOrigin = nullptr;
+  int32_t *m_dSlotTree = nullptr;
+  double *m_dPartial = nullptr;
+  size_t m_partialBytes = 0;
+  float *m_dStageIn = nullptr;
+  void *m_dStageOut = nullptr;
+  int64_t m_lastKernelMicros = 0;
+};
+
+} // namespace tbamd

@@ -1,0 +1,99 @@
+"""ctypes declarations for libtreebeard_amd.so (include/tbruntime_amd.h).
+
+Counterpart of the reference's `TreebeardAPI` (src/python/treebeard_runtime_api.py:12-…):
+loads the runtime library that sits next to this file and declares argument and
+return types of every entry point.  There is no fallback: a missing library is
+an error.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtreebeard_amd.so")
+
+c_i32, c_i64, c_ip, c_vp, c_cp = ctypes.c_int32, ctypes.c_int64, ctypes.c_ssize_t, ctypes.c_void_p, ctypes.c_char_p
+
+OPTION_SETTERS = ["numberOfFeatures", "batchSize", "tileSize", "thresholdTypeWidth", "returnTypeWidth",
+                  "returnTypeFloatType", "featureIndexTypeWidth", "nodeIndexTypeWidth", "inputElementTypeWidth",
+                  "tileShapeBitWidth", "childIndexBitWidth", "makeAllLeavesSameDepth", "reorderTreesByDepth",
+                  "pipelineSize", "numberOfCores", "numParallelTreeBatches", "tilingType"]
+GPU_OPTION_SETTERS = ["numRowsPerTB", "numRowsPerThread", "rowTileSize", "numTreeThreads", "numTreesAtATime",
+                      "cacheRows", "cacheTrees", "unrollTreeWalks", "treeWalkInterleaveFactor", "sharedMemoryReduce"]
+
+SIGNATURES = {
+    "RunInference": (None, [c_ip, c_vp, c_vp]),
+    "RunInferenceOnMultipleBatches": (None, [c_ip, c_vp, c_vp, c_i32]),
+    "GetBatchSize": (c_i32, [c_ip]),
+    "GetRowSize": (c_i32, [c_ip]),
+    "DeleteInferenceRunner": (None, [c_ip]),
+    "CreateCompilerOptions": (c_ip, []),
+    "DeleteCompilerOptions": (None, [c_ip]),
+    "Set_statsProfileCSVPath": (None, [c_ip, c_cp]),
+    "CreateGPUAutoScheduleOptions": (c_ip, []),
+    "DeleteGPUAutoScheduleOptions": (None, [c_ip]),
+    "CreateInferenceRunner": (c_ip, [c_cp, c_cp, c_ip]),
+    "CreateInferenceRunnerForONNXModel": (c_ip, [c_cp, c_ip]),
+    "SetEnableSparseRepresentation": (None, [c_i32]),
+    "IsSparseRepresentationEnabled": (c_i32, []),
+    "SetPeeledCodeGenForProbabilityBasedTiling": (None, [c_i32]),
+    "IsPeeledCodeGenForProbabilityBasedTilingEnabled": (c_i32, []),
+    "SetEnableMeasureGpuKernelTime": (None, [ctypes.c_bool]),
+    "SetNumberOfKernelRuns": (None, [c_i32]),
+    "GetGPUKernelExecutionTime": (c_i64, [c_ip]),
+    "ConstructTreebeardContext": (c_ip, [c_cp, c_cp, c_ip]),
+    "ConstructTreebeardContextFromGPUAutoscheduleOptions": (c_ip, [c_cp, c_cp, c_ip, c_ip]),
+    "DestroyTreebeardContext": (None, [c_ip]),
+    "SetForestCreatorType": (None, [c_ip, c_cp]),
+    "SetRepresentationAndSerializer": (None, [c_ip, c_cp]),
+    "ConstructGPUInferenceRunnerFromTBContext": (c_vp, [c_vp]),
+    "ConstructInferenceRunnerFromHIR": (c_vp, [c_vp]),
+    "ConstructGPUInferenceRunnerFromHIR": (c_vp, [c_vp]),
+    "BuildHIRRepresentation": (None, [c_vp]),
+    "findBestGPUScheduleAndCompileModel": (c_vp, [c_vp]),
+    "tbmi_last_error": (c_cp, []),
+    "tbmi_device_count": (c_i32, []),
+    "tbmi_run_device": (c_i32, [c_ip, c_vp, c_vp, c_i64]),
+    "tbmi_run_device_multiclass": (c_i32, [c_ip, c_vp, c_i64, c_vp, c_vp, c_vp]),
+    "tbmi_dump_leaf_ids": (c_i32, [c_ip, c_vp, c_vp, c_i64]),
+    "tbmi_time_kernels": (c_i32, [c_ip, c_vp, c_vp, c_i64, c_i32, ctypes.POINTER(ctypes.c_double),
+                                  ctypes.POINTER(ctypes.c_double)]),
+    "tbmi_autotune": (c_i32, [c_ip, c_vp, c_i64, ctypes.POINTER(ctypes.c_double)]),
+    "tbmi_set_plan": (c_i32, [c_ip, c_i32, c_i32, c_i32, c_i32]),
+    "tbmi_describe_plan": (c_i32, [c_ip, c_cp, c_i32]),
+    "tbmi_num_trees": (c_i32, [c_ip]),
+    "tbmi_num_classes": (c_i32, [c_ip]),
+    "tbmi_load_forest": (c_ip, [c_cp, c_cp, c_i32]),
+    "tbmi_delete_forest": (None, [c_ip]),
+    "tbmi_forest_info": (c_i32, [c_ip, ctypes.POINTER(c_i64), ctypes.POINTER(ctypes.c_double)]),
+    "tbmi_forest_tree_size": (c_i32, [c_ip, c_i32]),
+    "tbmi_forest_tree": (c_i32, [c_ip, c_i32, c_vp, c_vp, c_vp, c_vp, ctypes.POINTER(c_i32)]),
+    "tbmi_pack_roundtrip": (c_i32, [c_ip, c_i32, c_i32, c_i32, ctypes.POINTER(c_i64)]),
+}
+for _name in OPTION_SETTERS + GPU_OPTION_SETTERS:
+    SIGNATURES["Set_" + _name] = (None, [c_ip, c_i32])
+
+
+class TreebeardAPI:
+    def __init__(self, lib_path=LIB_PATH):
+        if not os.path.exists(lib_path):
+            raise FileNotFoundError(
+                "%s is missing: build it with `python -m treebeard_amd.build` (there is no fallback path)" % lib_path)
+        self.runtime_lib = ctypes.CDLL(lib_path)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(self.runtime_lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+
+    def last_error(self):
+        msg = self.runtime_lib.tbmi_last_error()
+        return msg.decode() if msg else ""
+
+
+_api = None
+
+
+def api():
+    global _api
+    if _api is None:
+        _api = TreebeardAPI()
+    return _api
