@@ -1,0 +1,125 @@
+#!/usr/bin/env python3
+"""Headline benchmark: rows/s of decision-forest inference on one MI355X.
+
+Workload: BASELINE.json configs[1] - 1000 trees, depth <= 8, 28 features,
+binary:logistic, 2^20-row batch, rows already resident in HBM.  One "step" is
+one pass of the hot path (walk kernel + output transform) over the batch.
+Prints ONE JSON line with the throughput, the roofline fractions of the walk
+kernel (measured live with HIP events on the runtime's own stream) and the CPU
+baseline (the oracle's multithreaded one-tree-at-a-time schedule) timed on the
+host cores on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0                      # MI355X HBM3E, published
+LDS_PEAK_GBS = 256 * 128 * 2.4             # 256 CUs x 128 B/clk x 2.4 GHz = 78 643 GB/s, nominal
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (default: the headline, 2)")
+    ap.add_argument("--rows", type=int, default=0, help="override the batch size")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--autotune", action="store_true", help="timed launch-plan search before measuring")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU-baseline duration")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this engine runs on ONE GPU (rows shard trivially; see DESIGN.md) - use --gpus 1")
+
+    import numpy as np
+    import torch
+
+    from treebeard_amd import synth, treebeard
+
+    cfg = synth.CONFIGS[args.config]
+    rows = args.rows or cfg.batch
+    cache = os.path.join(tempfile.gettempdir(), "treebeard_amd_models")
+    model = synth.model_path(args.config, cache)
+    x = cfg.batch_rows(rows)
+    runner = treebeard.TreebeardInferenceRunner.FromModelFile(model, "", treebeard.CompilerOptions(rows, 1))
+    multiclass = runner.num_classes() > 0
+    dx = torch.from_numpy(x).cuda()
+    out = torch.zeros(rows, dtype=torch.int8 if multiclass else torch.float32, device="cuda")
+    if args.autotune:
+        runner.autotune(dx.data_ptr(), rows)
+
+    for _ in range(args.warmup):
+        runner.run_device(dx.data_ptr(), out.data_ptr(), rows)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        runner.run_device(dx.data_ptr(), out.data_ptr(), rows)      # synchronises the runtime's stream
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    rows_per_s = rows / (elapsed / args.steps)
+
+    # kernel-only duration of the dominant (walk) kernel: HIP events on the stream it is launched on
+    walk_ms, fin_ms = runner.time_kernels(dx.data_ptr(), out.data_ptr(), rows, max(args.steps, 5))
+
+    # algorithmic bytes per row: HBM = 4 F + output; LDS = visited internal nodes x 6 B + 4 B per leaf,
+    # the visit count measured exactly by the oracle on a sample of the same rows
+    from oracle import cpu_oracle, model_io
+    forest = model_io.load_xgboost_json(model)
+    sample = min(rows, 8192)
+    steps_per_row = cpu_oracle.total_steps(forest, x[:sample]) / sample
+    hbm_bytes_row = 4 * cfg.num_features + (1 if multiclass else 4)
+    lds_bytes_row = steps_per_row * 6 + 4 * forest.num_trees
+    hbm_gbs = hbm_bytes_row * rows / (walk_ms * 1e-3) / 1e9
+    lds_gbs = lds_bytes_row * rows / (walk_ms * 1e-3) / 1e9
+    hbm_time = hbm_bytes_row * rows / (HBM_PEAK_GBS * 1e9)
+    lds_time = lds_bytes_row * rows / (LDS_PEAK_GBS * 1e9)
+    binding = "lds" if lds_time > hbm_time else "hbm"
+
+    line = {
+        "metric": "rows/sec at 1 MI355X (2^20-row batch) + % of binding HBM/LDS roofline",
+        "value": rows_per_s, "unit": "rows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": cfg.name, "rows": rows, "trees": forest.num_trees, "features": cfg.num_features,
+                   "objective": cfg.objective, "plan": runner.describe_plan()},
+        "roofline": {"bound": "hbm", "achieved": hbm_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": hbm_gbs / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "WalkRowsLdsKernel" if "rows_lds" in runner.describe_plan() else "WalkTreeParallelKernel",
+                     "kernel_ms": walk_ms, "finalize_ms": fin_ms, "algorithmic_bytes_per_row": hbm_bytes_row},
+        "roofline_binding": {"bound": binding, "achieved": lds_gbs if binding == "lds" else hbm_gbs,
+                             "peak": LDS_PEAK_GBS if binding == "lds" else HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": (lds_gbs / LDS_PEAK_GBS) if binding == "lds" else (hbm_gbs / HBM_PEAK_GBS),
+                             "algorithmic_bytes_per_row": lds_bytes_row if binding == "lds" else hbm_bytes_row,
+                             "visited_nodes_per_row": steps_per_row,
+                             "peak_note": "nominal LDS bandwidth 256 CUs x 128 B/clk x 2.4 GHz"},
+    }
+
+    if not args.no_cpu_baseline:
+        threads = cpu_oracle.max_threads()
+        order = np.argsort([forest.depth(t) for t in range(forest.num_trees)], kind="stable").astype(np.int32)
+        probe = min(rows, 2048)
+        t0 = time.perf_counter()
+        cpu_oracle.predict_tree_outer(forest, x[:probe], tree_order=order, threads=threads)
+        per_row = (time.perf_counter() - t0) / probe
+        cpu_rows = int(min(rows, max(probe, args.cpu_seconds / max(per_row, 1e-9))))
+        t0 = time.perf_counter()
+        cpu_out = cpu_oracle.predict_tree_outer(forest, x[:cpu_rows], tree_order=order, threads=threads)
+        cpu_s = time.perf_counter() - t0
+        line["cpu_baseline"] = {"value": cpu_rows / cpu_s, "unit": "rows/s", "cores": threads, "kind": "port",
+                                "sample": "first %d rows of the same batch, one-tree-at-a-time schedule, batch split "
+                                          "over %d threads, scalar walk (tile size 1)" % (cpu_rows, threads)}
+        if not multiclass:
+            got = out[:cpu_rows].cpu().numpy()
+            line["cpu_baseline"]["max_abs_diff_vs_gpu"] = float(np.abs(got - cpu_out).max())
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

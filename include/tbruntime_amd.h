@@ -129,6 +129,9 @@ TBAMD_EXPORT int32_t tbmi_autotune(intptr_t runner, const float *deviceInputs, i
 /* Pins a launch plan (values <= 0 keep the current one). */
 TBAMD_EXPORT int32_t tbmi_set_plan(intptr_t runner, int32_t rowsPerBlock, int32_t interleave, int32_t groupBytes,
                                    int32_t treeSlices);
+/* Pins the tree-parallel kernel: rowsPerBlock rows per block, treeLanes lanes per row. */
+TBAMD_EXPORT int32_t tbmi_set_tree_parallel_plan(intptr_t runner, int32_t rowsPerBlock, int32_t treeLanes,
+                                                 int32_t interleave, int32_t groupBytes, int32_t treeSlices);
 TBAMD_EXPORT int32_t tbmi_describe_plan(intptr_t runner, char *buffer, int32_t length);
 TBAMD_EXPORT int32_t tbmi_num_trees(intptr_t runner);
 TBAMD_EXPORT int32_t tbmi_num_classes(intptr_t runner);

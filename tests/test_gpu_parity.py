@@ -1,0 +1,296 @@
+"""Parity of the HIP path with the CPU oracle, through the C ABI, on a real GPU.
+
+Bars: per-tree leaf selection bit-exact; predictions within 1e-5 relative of the
+oracle (sums) and 1e-6 absolute (sigmoid / softmax); class ids equal.  At the
+full benchmark sizes, where the oracle would take minutes, the checks are
+size-independent properties (sub-batch consistency, permutation equivariance)
+plus an oracle comparison on a random sample of rows.
+"""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+from oracle import cpu_oracle, model_io  # noqa: E402
+from treebeard_amd import synth, treebeard  # noqa: E402
+from treebeard_amd.runtime_api import api  # noqa: E402
+
+from conftest import BENCHMARK_XGB, GOLDEN, benchmark_csv, benchmark_model, random_models  # noqa: E402
+from onnx_writer import write_onnx  # noqa: E402
+
+RTOL_SUM = 1e-5
+ATOL_PROB = 1e-6
+
+
+@pytest.fixture(scope="module", autouse=True)
+def require_gpu():
+    assert api().runtime_lib.tbmi_device_count() >= 1, "the GPU tests need a HIP device"
+    assert torch.cuda.is_available()
+
+
+def make_runner(path, batch, kind="xgboost_json", num_features=0, gpu_options=None):
+    options = treebeard.CompilerOptions(batch, 1)
+    if num_features:
+        options.SetNumberOfFeatures(num_features)
+    ctx = treebeard.TreebeardContext(str(path), "", options, gpu_options)
+    ctx.SetInputFiletype(kind)
+    ctx.SetRepresentationType("gpu_sparse")
+    return treebeard.TreebeardInferenceRunner.GPUInferenceRunnerFromTBContext(ctx)
+
+
+def gpu_predict(runner, x):
+    dx = torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).cuda()
+    rows = x.shape[0]
+    if runner.num_classes() > 0:
+        out = torch.full((rows,), -1, dtype=torch.int8, device="cuda")
+    else:
+        out = torch.full((rows,), float("nan"), dtype=torch.float32, device="cuda")
+    runner.run_device(dx.data_ptr(), out.data_ptr(), rows)
+    return out.cpu().numpy()
+
+
+def gpu_leaf_ids(runner, x):
+    dx = torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).cuda()
+    ids = torch.full((x.shape[0], runner.num_trees()), -7, dtype=torch.int32, device="cuda")
+    runner.dump_leaf_ids(dx.data_ptr(), ids.data_ptr(), x.shape[0])
+    return ids.cpu().numpy()
+
+
+def check_against_oracle(runner, forest, x):
+    np.testing.assert_array_equal(gpu_leaf_ids(runner, x), cpu_oracle.leaf_ids(forest, x))
+    pred, sums = cpu_oracle.predict(forest, x)
+    got = gpu_predict(runner, x)
+    if forest.num_classes > 0:
+        np.testing.assert_array_equal(got.astype(np.float32), pred)
+    elif forest.transform == model_io.SIGMOID:
+        np.testing.assert_allclose(got, pred, rtol=0, atol=ATOL_PROB)
+    else:
+        np.testing.assert_allclose(got, pred, rtol=RTOL_SUM, atol=0)
+    return got
+
+
+# --------------------------------------------------------------------------
+# the reference's own fixtures
+# --------------------------------------------------------------------------
+@pytest.mark.parametrize("path", random_models(), ids=os.path.basename)
+def test_random_models(path):
+    forest = model_io.load_xgboost_json(path)
+    x, expected = model_io.read_csv(path + ".csv")
+    x = x.astype(np.float32)
+    runner = make_runner(path, x.shape[0])
+    got = check_against_oracle(runner, forest, x)
+    np.testing.assert_allclose(got, expected, rtol=2e-5, atol=2e-5)   # XGBoost's own f32-accumulated output
+    # host-buffer entry point, as the reference's tests drive it (batch = whole CSV)
+    np.testing.assert_array_equal(runner.RunInference(x), got)
+
+
+@pytest.mark.parametrize("name", BENCHMARK_XGB)
+def test_benchmark_models(name, plain_file):
+    forest = model_io.load_xgboost_json(benchmark_model(name))
+    x, expected = model_io.read_csv(benchmark_csv(name))
+    x = x.astype(np.float32)
+    runner = make_runner(plain_file(benchmark_model(name)), 100)
+    got = check_against_oracle(runner, forest, x)
+    if forest.transform == model_io.SIGMOID:
+        np.testing.assert_allclose(got, expected, rtol=0, atol=ATOL_PROB)
+    else:
+        np.testing.assert_allclose(got, expected, rtol=RTOL_SUM, atol=0)
+    # 200 rows = 2 batches of 100 (the reference's python tests feed fixed batches)
+    np.testing.assert_array_equal(runner.RunInferenceOnMultipleBatches(x), got)
+
+
+def test_onnx_abalone(plain_file):
+    path = os.path.join(GOLDEN, "benchmark", "abalone_onnx_model_save.onnx.gz")
+    forest = model_io.load_onnx(path, 8)
+    x, expected = model_io.read_csv(os.path.join(GOLDEN, "benchmark", "abalone_onnx_model_save.onnx.csv"))
+    x = x.astype(np.float32)
+    options = treebeard.CompilerOptions(x.shape[0], 1)
+    options.SetNumberOfFeatures(8)
+    runner = treebeard.TreebeardInferenceRunner.FromONNXModelFile(plain_file(path), options)
+    got = check_against_oracle(runner, forest, x)
+    np.testing.assert_allclose(got, expected, rtol=RTOL_SUM, atol=0)
+
+
+@pytest.mark.parametrize("mode", ["BRANCH_LT", "BRANCH_GEQ", "BRANCH_GT", "BRANCH_LEQ"])
+def test_onnx_comparison_modes(tmp_path, mode):
+    rng = np.random.default_rng(11)
+    trees = []
+    for _ in range(9):
+        thr = rng.integers(-3, 4, size=7).astype(np.float32) / 2      # coarse grid: x == threshold happens
+        trees.append((thr, rng.integers(0, 4, 7), [1, 3, 5, -1, -1, -1, -1], [2, 4, 6, -1, -1, -1, -1]))
+    path = tmp_path / "m.onnx"
+    write_onnx(path, trees, mode=mode, base_value=0.5)
+    forest = model_io.load_onnx(path, 4)
+    x = (rng.integers(-4, 5, size=(777, 4)) / 2).astype(np.float32)
+    runner = make_runner(path, 777, "onnx_file", 4)
+    check_against_oracle(runner, forest, x)
+
+
+# --------------------------------------------------------------------------
+# the benchmark configurations at oracle-sized batches
+# --------------------------------------------------------------------------
+@pytest.mark.parametrize("k,rows", [(1, 1024), (2, 4096), (3, 4096), (4, 512), (5, 4096)])
+def test_synthetic_configurations(synth_model, k, rows):
+    forest = model_io.load_xgboost_json(synth_model(k))
+    x = synth.CONFIGS[k].batch_rows(rows)
+    runner = make_runner(synth_model(k), rows)
+    check_against_oracle(runner, forest, x)
+    if k == 3:
+        dx = torch.from_numpy(x).cuda()
+        cls = torch.zeros(rows, dtype=torch.int8, device="cuda")
+        margins = torch.zeros((rows, 8), dtype=torch.float32, device="cuda")
+        probs = torch.zeros((rows, 8), dtype=torch.float32, device="cuda")
+        runner.run_device_multiclass(dx.data_ptr(), rows, cls.data_ptr(), margins.data_ptr(), probs.data_ptr())
+        pred, sums = cpu_oracle.predict(forest, x)
+        np.testing.assert_allclose(margins.cpu().numpy(), sums, rtol=RTOL_SUM, atol=1e-7)
+        # softmax probabilities: closed form only (the reference never computes them)
+        np.testing.assert_allclose(probs.cpu().numpy(), cpu_oracle.softmax(sums), rtol=0, atol=ATOL_PROB)
+        np.testing.assert_array_equal(cls.cpu().numpy(), cpu_oracle.argmax_generated(sums.astype(np.float32)))
+
+
+@pytest.mark.parametrize("rows", [1, 64, 4096, 1 << 16])
+def test_config2_batch_sweep(synth_model, rows):
+    forest = model_io.load_xgboost_json(synth_model(2))
+    x = synth.CONFIGS[2].batch_rows(rows, seed_offset=rows)
+    runner = make_runner(synth_model(2), rows)
+    if rows <= 4096:
+        check_against_oracle(runner, forest, x)
+    else:
+        pred, _ = cpu_oracle.predict(forest, x)
+        np.testing.assert_allclose(gpu_predict(runner, x), pred, rtol=0, atol=ATOL_PROB)
+
+
+@pytest.mark.parametrize("k", [2, 3, 5])
+def test_full_size_properties(synth_model, k):
+    cfg = synth.CONFIGS[k]
+    rows = cfg.batch
+    forest = model_io.load_xgboost_json(synth_model(k))
+    x = cfg.batch_rows(rows)
+    runner = make_runner(synth_model(k), rows)
+    full = gpu_predict(runner, x)
+    assert not np.isnan(full.astype(np.float32)).any()
+    rng = np.random.default_rng(k)
+    # (1) a random sample of rows against the oracle
+    pick = rng.choice(rows, size=4096, replace=False)
+    pred, _ = cpu_oracle.predict(forest, x[pick])
+    if forest.num_classes > 0:
+        np.testing.assert_array_equal(full[pick].astype(np.float32), pred)
+    elif forest.transform == model_io.SIGMOID:
+        np.testing.assert_allclose(full[pick], pred, rtol=0, atol=ATOL_PROB)
+    else:
+        np.testing.assert_allclose(full[pick], pred, rtol=RTOL_SUM, atol=0)
+    # (2) rows are independent: a ragged slice alone gives the same bits as inside the batch
+    lo, hi = 12345, 12345 + 70001
+    np.testing.assert_array_equal(gpu_predict(runner, x[lo:hi]), full[lo:hi])
+    # (3) permutation equivariance
+    perm = rng.permutation(rows)
+    np.testing.assert_array_equal(gpu_predict(runner, x[perm]), full[perm])
+
+
+# --------------------------------------------------------------------------
+# launch plans, edge cases, API behaviour
+# --------------------------------------------------------------------------
+@pytest.mark.parametrize("plan", [(64, 1, 16384, 1), (128, 2, 32768, 3), (256, 8, 65536, 1), (512, 4, 49152, 5),
+                                  (256, 4, 8192, 40)])
+def test_launch_plans_agree(synth_model, plan):
+    forest = model_io.load_xgboost_json(synth_model(2))
+    x = synth.CONFIGS[2].batch_rows(3001, seed_offset=9)
+    runner = make_runner(synth_model(2), 3001)
+    runner.set_plan(*plan)
+    assert "kernel=rows_lds rowsPerBlock=%d treeLanes=1 interleave=%d" % plan[:2] in runner.describe_plan()
+    check_against_oracle(runner, forest, x)
+
+
+@pytest.mark.parametrize("plan", [(1, 256, 1, 0, 0), (4, 64, 1, 32768, 7), (16, 16, 2, 0, 1), (2, 128, 1, 16384, 0),
+                                  (8, 8, 4, 0, 3), (64, 1, 1, 0, 2), (1, 1024, 1, 65536, 1)])
+@pytest.mark.parametrize("k", [2, 3])
+def test_tree_parallel_plans_agree(synth_model, k, plan):
+    forest = model_io.load_xgboost_json(synth_model(k))
+    x = synth.CONFIGS[k].batch_rows(203, seed_offset=3)
+    runner = make_runner(synth_model(k), 203)
+    runner.set_tree_parallel_plan(*plan)
+    assert "kernel=tree_parallel rowsPerBlock=%d treeLanes=%d" % plan[:2] in runner.describe_plan()
+    check_against_oracle(runner, forest, x)
+
+
+@pytest.mark.parametrize("k,rows", [(3, 100), (5, 7), (1, 1)])
+def test_small_batches_pick_the_tree_parallel_kernel(synth_model, k, rows):
+    forest = model_io.load_xgboost_json(synth_model(k))
+    x = synth.CONFIGS[k].batch_rows(rows, seed_offset=1)
+    runner = make_runner(synth_model(k), rows)
+    assert "kernel=tree_parallel" in runner.describe_plan()
+    check_against_oracle(runner, forest, x)
+
+
+def test_gpu_auto_schedule_options_are_honoured(synth_model):
+    gpu = treebeard.GPUAutoScheduleOptions.Construct(num_rows_per_TB=64, num_tree_threads=10,
+                                                     tree_walk_interleave_factor=2, cache_rows=True)
+    runner = make_runner(synth_model(1), 1024, gpu_options=gpu)
+    plan = runner.describe_plan()
+    assert "kernel=rows_lds rowsPerBlock=64 " in plan and "interleave=2" in plan
+    forest = model_io.load_xgboost_json(synth_model(1))
+    check_against_oracle(runner, forest, synth.CONFIGS[1].batch_rows(1024))
+
+
+def test_autotuned_runner_matches(synth_model):
+    options = treebeard.CompilerOptions(8192, 1)
+    ctx = treebeard.TreebeardContext(synth_model(1), "", options)
+    runner = treebeard.TreebeardInferenceRunner.AutoScheduleGPUInferenceRunnerFromTBContext(ctx)
+    forest = model_io.load_xgboost_json(synth_model(1))
+    check_against_oracle(runner, forest, synth.CONFIGS[1].batch_rows(8192))
+
+
+def test_degenerate_models(tmp_path):
+    rng = np.random.Generator(np.random.PCG64(4))
+    stump = synth._grow_tree(rng, 0, lambda d, s: 0.0, lambda: (0, 0.0), lambda: 0.75, force_root=False)   # single leaf
+    deep = synth._grow_tree(rng, 9, lambda d, s: 1.0 if s <= 0 else 0.0, lambda: (rng.integers(0, 3), rng.normal()),
+                            lambda: rng.normal())                                                         # left spine
+    one = synth._grow_tree(rng, 1, lambda d, s: 1.0, lambda: (1, 0.0), lambda: rng.normal())
+    for name, trees in (("stump", [stump]), ("mixed", [stump, deep, one, stump]), ("one", [one])):
+        path = tmp_path / (name + ".json")
+        synth.write_xgboost_json(path, trees, 3)
+        forest = model_io.load_xgboost_json(path)
+        x = rng.normal(size=(130, 3)).astype(np.float32)
+        x[5, 1] = 0.0          # equal to a threshold
+        x[7, :] = np.inf
+        x[8, :] = -np.inf
+        check_against_oracle(make_runner(path, 130), forest, x)
+
+
+def test_zero_rows_and_errors(synth_model):
+    runner = make_runner(synth_model(1), 16)
+    runner.run_device(None, None, 0)
+    lib = api().runtime_lib
+    assert lib.tbmi_run_device(0, None, None, 4) == -1 and "null" in api().last_error()
+    options = treebeard.CompilerOptions(16, 1)
+    options.SetInputElementTypeWidth(64)
+    with pytest.raises(RuntimeError, match="32-bit float inputs"):
+        treebeard.TreebeardInferenceRunner.FromModelFile(synth_model(1), "", options)
+    with pytest.raises(RuntimeError, match="cannot open"):
+        treebeard.TreebeardInferenceRunner.FromModelFile("/nonexistent.json", "", treebeard.CompilerOptions(16, 1))
+
+
+def test_kernel_time_shim(synth_model):
+    runner = make_runner(synth_model(1), 1024)
+    x = synth.CONFIGS[1].batch_rows(1024)
+    treebeard.SetEnableMeasureGpuKernelTime(True)
+    treebeard.SetNumberOfKernelRuns(10)
+    try:
+        runner.RunInference(x)
+        ten = treebeard.GetGPUKernelExecutionTime(runner)
+        treebeard.SetNumberOfKernelRuns(1)
+        runner.RunInference(x)
+        one = treebeard.GetGPUKernelExecutionTime(runner)
+    finally:
+        treebeard.SetEnableMeasureGpuKernelTime(False)
+        treebeard.SetNumberOfKernelRuns(1)
+    assert ten > one > 0
+    dx = torch.from_numpy(x).cuda()
+    out = torch.zeros(1024, dtype=torch.float32, device="cuda")
+    walk_ms, fin_ms = runner.time_kernels(dx.data_ptr(), out.data_ptr(), 1024, 5)
+    assert 0 < walk_ms < 50 and fin_ms >= 0

@@ -1,0 +1,193 @@
+"""Host-side logic of the runtime library, runnable without a GPU: the C-ABI
+exports everything include/tbruntime_amd.h declares, the C++ loaders build the
+same forests as the oracle's loaders, packing round-trips, and errors come
+back as messages instead of aborts (the reference asserts,
+src/json/xgboostparser.h:100, src/runtime/runtime.cpp:172)."""
+import ctypes
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+
+from oracle import model_io
+from treebeard_amd import runtime_api, synth
+
+from conftest import BENCHMARK_XGB, GOLDEN, ROOT, benchmark_model, random_models
+from onnx_writer import write_onnx
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return runtime_api.api().runtime_lib
+
+
+def last_error():
+    return runtime_api.api().last_error()
+
+
+def load_forest(lib, path, kind="xgboost_json", num_features=0):
+    h = lib.tbmi_load_forest(str(path).encode(), kind.encode(), num_features)
+    assert h, last_error()
+    return h
+
+
+def forest_arrays(lib, h):
+    info = (ctypes.c_int64 * 6)()
+    init = ctypes.c_double()
+    assert lib.tbmi_forest_info(h, info, ctypes.byref(init)) == 0
+    trees = []
+    for t in range(info[0]):
+        n = lib.tbmi_forest_tree_size(h, t)
+        v, f = np.empty(n, np.float32), np.empty(n, np.int32)
+        l, r = np.empty(n, np.int32), np.empty(n, np.int32)
+        c = ctypes.c_int32()
+        assert lib.tbmi_forest_tree(h, t, v.ctypes.data, f.ctypes.data, l.ctypes.data, r.ctypes.data, ctypes.byref(c)) == 0
+        trees.append((v, f, l, r, c.value))
+    return list(info), init.value, trees
+
+
+def assert_same_forest(lib, h, forest):
+    info, init, trees = forest_arrays(lib, h)
+    assert info[:5] == [forest.num_trees, forest.num_features, forest.num_classes, forest.transform, forest.predicate]
+    assert info[5] == len(forest.threshold)
+    assert init == forest.initial_value
+    for t, (v, f, l, r, c) in enumerate(trees):
+        thr, feat, left, right = forest.tree(t)
+        np.testing.assert_array_equal(v.astype(np.float64), thr)
+        np.testing.assert_array_equal(l, left)
+        np.testing.assert_array_equal(r, right)
+        internal = left != -1
+        np.testing.assert_array_equal(f[internal], feat[internal])
+        assert c == forest.class_id[t]
+
+
+def test_every_declared_symbol_is_exported(lib):
+    header = open(os.path.join(ROOT, "include", "tbruntime_amd.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    header = header.replace("#define TBAMD_EXPORT", "")
+    names = re.findall(r"TBAMD_EXPORT\s+[^;(]*?\b(\w+)\s*\(", header)
+    assert len(names) > 70
+    for name in names:
+        assert hasattr(lib, name), name
+    assert set(runtime_api.SIGNATURES) == set(names)
+
+
+@pytest.mark.parametrize("path", random_models()[::2] + [benchmark_model(n) for n in BENCHMARK_XGB], ids=os.path.basename)
+def test_xgboost_loader_matches_oracle_loader(lib, plain_file, path):
+    h = load_forest(lib, plain_file(path))
+    assert_same_forest(lib, h, model_io.load_xgboost_json(path))
+    lib.tbmi_delete_forest(h)
+
+
+@pytest.mark.parametrize("k", [1, 2, 3, 5])
+def test_synthetic_models_load_and_pack(lib, synth_model, k):
+    path = synth_model(k)
+    h = load_forest(lib, path)
+    assert_same_forest(lib, h, model_io.load_xgboost_json(path))
+    stats = (ctypes.c_int64 * 5)()
+    for rows_per_block, interleave, group_bytes in [(256, 4, 49152), (128, 8, 65536), (64, 1, 32768), (256, 2, 16384)]:
+        assert lib.tbmi_pack_roundtrip(h, rows_per_block, interleave, group_bytes, stats) == 0, last_error()
+        assert stats[3] <= 160 * 1024
+    lib.tbmi_delete_forest(h)
+
+
+def test_onnx_loader_matches_oracle_loader(lib, plain_file):
+    path = os.path.join(GOLDEN, "benchmark", "abalone_onnx_model_save.onnx.gz")
+    h = load_forest(lib, plain_file(path), "onnx_file", 8)
+    assert_same_forest(lib, h, model_io.load_onnx(path, 8))
+    lib.tbmi_delete_forest(h)
+
+
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("mode", ["BRANCH_LT", "BRANCH_GEQ", "BRANCH_GT", "BRANCH_LEQ"])
+def test_onnx_comparison_modes_and_encodings(lib, tmp_path, mode, packed):
+    rng = np.random.default_rng(3)
+    trees = [(rng.normal(size=7).astype(np.float32), rng.integers(0, 4, 7), [1, 3, 5, -1, -1, -1, -1], [2, 4, 6, -1, -1, -1, -1])
+             for _ in range(5)]
+    path = tmp_path / "m.onnx"
+    write_onnx(path, trees, mode=mode, base_value=0.25, packed=packed)
+    forest = model_io.load_onnx(path, 4)
+    assert forest.predicate == ["BRANCH_LT", "BRANCH_GEQ", "BRANCH_GT", "BRANCH_LEQ"].index(mode)
+    h = load_forest(lib, path, "onnx_file", 4)
+    assert_same_forest(lib, h, forest)
+    stats = (ctypes.c_int64 * 5)()
+    assert lib.tbmi_pack_roundtrip(h, 64, 2, 4096, stats) == 0, last_error()
+    lib.tbmi_delete_forest(h)
+
+
+def test_pack_rejects_plans_that_cannot_hold_the_model(lib, synth_model):
+    h = load_forest(lib, synth_model(5))
+    stats = (ctypes.c_int64 * 5)()
+    assert lib.tbmi_pack_roundtrip(h, 256, 4, 1024, stats) == -1      # deepest tree > one group
+    assert "does not fit" in last_error()
+    assert lib.tbmi_pack_roundtrip(h, 256, 3, 65536, stats) == -1     # interleave not a power of two
+    assert lib.tbmi_pack_roundtrip(h, 1024, 4, 65536, stats) == -1    # 16-bit feature offsets overflow
+    assert "16 bits" in last_error()
+    lib.tbmi_delete_forest(h)
+
+
+def test_loader_errors_are_reported_not_fatal(lib, tmp_path):
+    assert lib.tbmi_load_forest(b"/nonexistent/model.json", b"xgboost_json", 0) == 0
+    assert "cannot open" in last_error()
+    bad = tmp_path / "bad.json"
+    bad.write_text("{\"learner\": ")
+    assert lib.tbmi_load_forest(str(bad).encode(), b"xgboost_json", 0) == 0
+    assert "JSON" in last_error()
+    # unknown objective (the reference asserts: src/json/xgboostparser.h:94-102)
+    rng = np.random.Generator(np.random.PCG64(1))
+    tree = synth._grow_tree(rng, 2, lambda d, s: 1.0, lambda: (0, 0.5), lambda: 1.0)
+    path = tmp_path / "obj.json"
+    synth.write_xgboost_json(path, [tree], 2, objective="rank:pairwise")
+    assert lib.tbmi_load_forest(str(path).encode(), b"xgboost_json", 0) == 0
+    assert "Unknown objective" in last_error()
+    # feature index outside the declared features
+    doc = json.load(open(path))
+    doc["learner"]["objective"]["name"] = "reg:squarederror"
+    doc["learner"]["gradient_booster"]["model"]["trees"][0]["split_indices"][0] = 9
+    path.write_text(json.dumps(doc))
+    assert lib.tbmi_load_forest(str(path).encode(), b"xgboost_json", 0) == 0
+    assert "feature index" in last_error()
+    assert lib.tbmi_load_forest(str(path).encode(), b"treelite", 0) == 0
+    assert "unknown forest creator" in last_error()
+    # ONNX needs the feature count from the options (src/json/onnxmodelparser.h:345-348)
+    assert lib.tbmi_load_forest(os.path.join(GOLDEN, "handbuilt", "x.onnx").encode(), b"onnx_file", 0) == 0
+    assert "Number of features" in last_error()
+
+
+def test_option_handles_and_switches(lib):
+    o = lib.CreateCompilerOptions()
+    for name in runtime_api.OPTION_SETTERS:
+        getattr(lib, "Set_" + name)(o, 1)
+    lib.Set_tilingType(o, 7)
+    assert "Invalid tiling type" in last_error()
+    lib.Set_statsProfileCSVPath(o, b"/tmp/profile.csv")
+    lib.DeleteCompilerOptions(o)
+    g = lib.CreateGPUAutoScheduleOptions()
+    for name in runtime_api.GPU_OPTION_SETTERS:
+        getattr(lib, "Set_" + name)(g, 2)
+    lib.DeleteGPUAutoScheduleOptions(g)
+    lib.SetEnableSparseRepresentation(1)
+    assert lib.IsSparseRepresentationEnabled() == 1
+    lib.SetEnableSparseRepresentation(0)
+    lib.SetPeeledCodeGenForProbabilityBasedTiling(1)
+    assert lib.IsPeeledCodeGenForProbabilityBasedTilingEnabled() == 1
+    lib.SetPeeledCodeGenForProbabilityBasedTiling(0)
+    assert lib.GetBatchSize(0) == -1 and "null" in last_error()
+
+
+def test_synthetic_configurations_have_the_stated_shape(synth_model):
+    f1 = model_io.load_xgboost_json(synth_model(1))
+    assert (f1.num_trees, f1.num_features, f1.transform, f1.initial_value) == (100, 8, model_io.IDENTITY, 0.5)
+    assert all(f1.depth(t) == 6 and len(f1.tree(t)[0]) == 127 for t in range(100))
+    f2 = model_io.load_xgboost_json(synth_model(2))
+    assert (f2.num_trees, f2.num_features, f2.transform, f2.initial_value) == (1000, 28, model_io.SIGMOID, 0.0)
+    assert max(f2.depth(t) for t in range(1000)) == 8
+    f3 = model_io.load_xgboost_json(synth_model(3))
+    assert (f3.num_trees, f3.num_features, f3.num_classes) == (800, 54, 8)
+    np.testing.assert_array_equal(f3.class_id, np.arange(800) % 8)
+    f5 = model_io.load_xgboost_json(synth_model(5))
+    assert (f5.num_trees, f5.num_features) == (800, 90) and max(f5.depth(t) for t in range(800)) == 12
+    x3 = synth.CONFIGS[3].batch_rows(2000)
+    assert set(np.unique(x3[:, 10:])) <= {0.0, 1.0} and 0.05 < x3[:, 10:].mean() < 0.15

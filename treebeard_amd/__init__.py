@@ -1,0 +1,1 @@
+"""MI355X-native decision-forest inference behind Treebeard's runtime surface."""

@@ -17,6 +17,8 @@ struct WalkScalars {
   uint32_t groupRegionBytes = 0; // LDS bytes reserved for one tree group (multiple of 16)
   int32_t transform = 0;         // 0 identity, 1 sigmoid
   int32_t numTrees = 0;
+  int32_t rowsPerBlock = 0;      // tree-parallel kernel: rows per block
+  int32_t treeLanes = 1;         // tree-parallel kernel: lanes per row (power of two)
   double initialValue = 0.0;
 };
 
@@ -51,6 +53,9 @@ struct FinalizeParams {
 // `featureOffsetInWords` selects how node feature offsets are scaled.
 hipError_t LaunchWalkRowsLds(const WalkParams &p, int rowsPerBlock, int interleave, bool featureOffsetInWords,
                              size_t ldsBytes, hipStream_t stream);
+// Tree-parallel walk: s.rowsPerBlock rows per block (row-major in LDS),
+// s.treeLanes lanes per row; block = rowsPerBlock * treeLanes lanes.
+hipError_t LaunchWalkTreeParallel(const WalkParams &p, int interleave, size_t ldsBytes, hipStream_t stream);
 hipError_t LaunchFinalize(const FinalizeParams &p, hipStream_t stream);
 
 } // namespace tbamd

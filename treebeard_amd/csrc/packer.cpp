@@ -23,13 +23,19 @@ Forest NormalizeToLessThan(const Forest &forest) {
   return out;
 }
 
-uint32_t PackedModel::PadFeatureOffset() const {
-  uint32_t words = (uint32_t)numFeatures * (uint32_t)plan.rowsPerBlock;
-  return plan.featureOffsetInWords ? words : words * 4u;
-}
+uint32_t PackedModel::PadFeatureOffset() const { return (uint32_t)numFeatures * plan.FeatureStride(); }
+
+size_t PackedModel::RowTileBytes() const { return (size_t)(numFeatures + 1) * plan.rowsPerBlock * 4; }
 
 size_t PackedModel::LdsBytes() const {
-  return (size_t)(numFeatures + 1) * plan.rowsPerBlock * 4 + (size_t)maxGroupNodes * kNodeBytes;
+  size_t bytes = RowTileBytes() + (size_t)GroupRegionBytes();
+  if (plan.kernel == LaunchPlan::Kernel::kTreeParallel) {
+    // cross-wave reduction scratch + per-row, per-class accumulators (doubles)
+    const size_t waves = (size_t)(plan.ThreadsPerBlock() + 63) / 64;
+    bytes = (bytes + 7) & ~(size_t)7;
+    bytes += waves * 8 + (size_t)plan.rowsPerBlock * (numClasses > 0 ? numClasses : 1) * 8;
+  }
+  return bytes;
 }
 
 namespace {
@@ -60,8 +66,15 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
   const Forest forest = NormalizeToLessThan(input);
   const int K = plan.interleave;
   if (K < 1 || K > kMaxInterleave || (K & (K - 1))) throw Error("interleave must be 1, 2, 4 or 8");
-  if (plan.rowsPerBlock < 64 || (plan.rowsPerBlock & (plan.rowsPerBlock - 1)) || plan.rowsPerBlock > 1024)
-    throw Error("rowsPerBlock must be a power of two in [64, 1024]");
+  if (plan.kernel == LaunchPlan::Kernel::kRowParallelLds) {
+    if (plan.rowsPerBlock < 64 || (plan.rowsPerBlock & (plan.rowsPerBlock - 1)) || plan.rowsPerBlock > 1024)
+      throw Error("rowsPerBlock must be a power of two in [64, 1024]");
+  } else {
+    if (plan.treeLanes < 1 || (plan.treeLanes & (plan.treeLanes - 1)) || plan.rowsPerBlock < 1 ||
+        plan.ThreadsPerBlock() > 1024 || plan.ThreadsPerBlock() % 64 != 0)
+      throw Error("tree-parallel plan needs a power-of-two treeLanes and a block of 64..1024 lanes");
+    if (plan.treeLanes < 64 && 64 % plan.treeLanes != 0) throw Error("treeLanes must divide 64");
+  }
   if (plan.groupBytes < 1024 || plan.groupBytes > 65536) throw Error("groupBytes must be in [1024, 65536]");
 
   PackedModel pm;
@@ -72,8 +85,7 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
   const uint64_t padOffset = pm.PadFeatureOffset();
   if (padOffset > 0xFFFFu)
     throw Error("feature offsets do not fit 16 bits for this rowsPerBlock / feature count");
-  const uint32_t featureStride = plan.featureOffsetInWords ? (uint32_t)plan.rowsPerBlock
-                                                           : (uint32_t)plan.rowsPerBlock * 4u;
+  const uint32_t featureStride = plan.FeatureStride();
   const uint32_t groupCapacity = (uint32_t)plan.groupBytes / kNodeBytes;
 
   // Order: class, then depth (the reference sorts by depth for its GPU schedules,
@@ -180,8 +192,7 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
 
 Tree UnpackTree(const PackedModel &pm, int32_t treeIndex) {
   const int K = pm.plan.interleave;
-  const uint32_t featureStride = pm.plan.featureOffsetInWords ? (uint32_t)pm.plan.rowsPerBlock
-                                                              : (uint32_t)pm.plan.rowsPerBlock * 4u;
+  const uint32_t featureStride = pm.plan.FeatureStride();
   for (const DeviceGroup &g : pm.groups)
     for (uint32_t bi = g.bundleBegin; bi < g.bundleBegin + g.bundleCount; ++bi)
       for (int k = 0; k < K; ++k) {

@@ -8,15 +8,31 @@
 
 namespace tbamd {
 
-// How the row-parallel LDS kernel is launched; chosen by the tuner.
+// How the kernels are launched; chosen by the tuner.
+//
+//  kRowParallelLds: one lane per row, rowsPerBlock lanes per block, the block's
+//    rows transposed in LDS, every lane walks all trees (K at a time).
+//  kTreeParallel:   rowsPerBlock rows per block kept row-major in LDS and
+//    treeLanes lanes per row that split the trees between them; per-row sums are
+//    reduced across lanes (wave shuffles, then LDS across waves).  For models
+//    whose rows are too wide to transpose into LDS and for batches too small to
+//    fill the chip with one lane per row.
 struct LaunchPlan {
   enum class Kernel : int32_t { kRowParallelLds = 0, kTreeParallel = 1 };
   Kernel kernel = Kernel::kRowParallelLds;
-  int32_t rowsPerBlock = 256;   // = threads per block (one row per lane), power of two
+  int32_t rowsPerBlock = 256;   // row-parallel: = threads per block, power of two
+  int32_t treeLanes = 1;        // tree-parallel: lanes per row, power of two; block = rowsPerBlock * treeLanes
   int32_t interleave = 4;       // K: trees walked concurrently by one lane (1, 2, 4, 8)
   int32_t groupBytes = 48 * 1024; // LDS bytes for one tree group's nodes (<= 65536)
   int32_t treeSlices = 1;       // grid.y: how many blocks share one row block's trees
   bool featureOffsetInWords = false;
+
+  int32_t ThreadsPerBlock() const { return kernel == Kernel::kTreeParallel ? rowsPerBlock * treeLanes : rowsPerBlock; }
+  // Distance in LDS between feature f and f+1 of one row, in the units node offsets use.
+  uint32_t FeatureStride() const {
+    if (kernel == Kernel::kTreeParallel) return 4u;
+    return featureOffsetInWords ? (uint32_t)rowsPerBlock : (uint32_t)rowsPerBlock * 4u;
+  }
 };
 
 struct PackedModel {
@@ -33,7 +49,9 @@ struct PackedModel {
   uint32_t maxGroupNodes = 0;
 
   uint32_t PadFeatureOffset() const;
-  size_t LdsBytes() const; // transposed row tile + the largest group
+  uint32_t GroupRegionBytes() const { return maxGroupNodes * kNodeBytes; }
+  size_t RowTileBytes() const;
+  size_t LdsBytes() const; // row tile + the largest group (+ reduction scratch)
 };
 
 // Throws tbamd::Error when the plan cannot hold the model (tree larger than a

@@ -111,6 +111,14 @@ void InferenceRunner::EnsureStaging() {
   Check(hipMalloc(&m_dStageOut, rows * sizeof(float)), "allocate output staging");
 }
 
+hipError_t InferenceRunner::LaunchWalk(const WalkParams &p) const {
+  const LaunchPlan &plan = m_model.plan;
+  if (plan.kernel == LaunchPlan::Kernel::kTreeParallel)
+    return LaunchWalkTreeParallel(p, plan.interleave, m_model.LdsBytes(), m_stream);
+  return LaunchWalkRowsLds(p, plan.rowsPerBlock, plan.interleave, plan.featureOffsetInWords, m_model.LdsBytes(),
+                           m_stream);
+}
+
 WalkParams InferenceRunner::MakeWalkParams(const float *deviceInputs, int64_t rows) const {
   WalkParams p;
   p.s.rows = rows;
@@ -121,6 +129,8 @@ WalkParams InferenceRunner::MakeWalkParams(const float *deviceInputs, int64_t ro
   p.s.groupRegionBytes = (uint32_t)m_model.maxGroupNodes * kNodeBytes;
   p.s.transform = m_forest.transform == Transform::kSigmoid ? 1 : 0;
   p.s.numTrees = (int32_t)m_forest.trees.size();
+  p.s.rowsPerBlock = m_model.plan.rowsPerBlock;
+  p.s.treeLanes = m_model.plan.treeLanes;
   p.s.initialValue = m_forest.initialValue;
   p.x = deviceInputs;
   p.nodes16 = reinterpret_cast<const uint4 *>(m_dNodes);
@@ -142,9 +152,7 @@ void InferenceRunner::Launch(const float *deviceInputs, int64_t rows, float *out
     p.nodeOrigin = m_dNodeOrigin;
     p.slotTree = m_dSlotTree;
   }
-  Check(LaunchWalkRowsLds(p, m_model.plan.rowsPerBlock, m_model.plan.interleave, m_model.plan.featureOffsetInWords,
-                          m_model.LdsBytes(), m_stream),
-        "launch walk kernel");
+  Check(LaunchWalk(p), "launch walk kernel");
   if (finalize) {
     FinalizeParams f;
     f.partial = m_dPartial;
@@ -218,10 +226,7 @@ void InferenceRunner::TimeKernels(const float *deviceInputs, void *deviceResults
   p.out = finalize ? nullptr : static_cast<float *>(deviceResults);
   p.partial = finalize ? m_dPartial : nullptr;
   Check(hipEventRecord(m_evStart, m_stream), "hipEventRecord");
-  for (int i = 0; i < runs; ++i)
-    Check(LaunchWalkRowsLds(p, m_model.plan.rowsPerBlock, m_model.plan.interleave, m_model.plan.featureOffsetInWords,
-                            m_model.LdsBytes(), m_stream),
-          "launch walk kernel");
+  for (int i = 0; i < runs; ++i) Check(LaunchWalk(p), "launch walk kernel");
   Check(hipEventRecord(m_evStop, m_stream), "hipEventRecord");
   Check(hipStreamSynchronize(m_stream), "walk kernel");
   float ms = 0.f;
@@ -280,7 +285,8 @@ double InferenceRunner::AutoTune(const float *deviceInputs, int64_t rows) {
 std::string InferenceRunner::DescribePlan() const {
   std::ostringstream os;
   const LaunchPlan &p = m_model.plan;
-  os << "kernel=rows_lds rowsPerBlock=" << p.rowsPerBlock << " interleave=" << p.interleave
+  os << "kernel=" << (p.kernel == LaunchPlan::Kernel::kTreeParallel ? "tree_parallel" : "rows_lds")
+     << " rowsPerBlock=" << p.rowsPerBlock << " treeLanes=" << p.treeLanes << " interleave=" << p.interleave
      << " groupBytes=" << p.groupBytes << " treeSlices=" << p.treeSlices
      << " offsetsInWords=" << (p.featureOffsetInWords ? 1 : 0) << " groups=" << m_model.groups.size()
      << " bundles=" << m_model.bundles.size() << " nodes=" << m_model.nodes.size()

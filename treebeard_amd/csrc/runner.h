@@ -68,6 +68,7 @@ private:
   void EnsureStaging();
   bool NeedsFinalize() const { return m_model.plan.treeSlices > 1 || m_forest.numClasses > 0; }
   WalkParams MakeWalkParams(const float *deviceInputs, int64_t rows) const;
+  hipError_t LaunchWalk(const WalkParams &p) const;
   void Launch(const float *deviceInputs, int64_t rows, float *out, int8_t *classOut, float *margins,
               float *probabilities, int32_t *leafIds);
 

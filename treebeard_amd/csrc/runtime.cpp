@@ -335,12 +335,33 @@ int32_t tbmi_set_plan(intptr_t h, int32_t rowsPerBlock, int32_t interleave, int3
       [&] {
         InferenceRunner *r = Runner(h);
         LaunchPlan plan = r->Model().plan;
+        plan.kernel = LaunchPlan::Kernel::kRowParallelLds;
+        plan.treeLanes = 1;
         if (rowsPerBlock > 0) plan.rowsPerBlock = rowsPerBlock;
         if (interleave > 0) plan.interleave = interleave;
         if (groupBytes > 0) plan.groupBytes = groupBytes;
         if (treeSlices > 0) plan.treeSlices = treeSlices;
         const int64_t words = (int64_t)(r->RowSize() + 1) * plan.rowsPerBlock;
         plan.featureOffsetInWords = words * 4 > 0xFFFF;
+        r->Repack(plan);
+        return 0;
+      },
+      -1);
+}
+
+int32_t tbmi_set_tree_parallel_plan(intptr_t h, int32_t rowsPerBlock, int32_t treeLanes, int32_t interleave,
+                                    int32_t groupBytes, int32_t treeSlices) {
+  return Guard(
+      [&] {
+        InferenceRunner *r = Runner(h);
+        LaunchPlan plan = r->Model().plan;
+        plan.kernel = LaunchPlan::Kernel::kTreeParallel;
+        plan.featureOffsetInWords = false;
+        plan.rowsPerBlock = rowsPerBlock;
+        plan.treeLanes = treeLanes;
+        plan.interleave = interleave > 0 ? interleave : 1;
+        if (groupBytes > 0) plan.groupBytes = groupBytes;
+        if (treeSlices > 0) plan.treeSlices = treeSlices;
         r->Repack(plan);
         return 0;
       },

@@ -36,8 +36,69 @@ void FitGroupBytes(LaunchPlan &plan, const Forest &forest, const DeviceLimits &l
 
 } // namespace
 
+namespace {
+
+int64_t BiggestTreeNodes(const Forest &forest) {
+  int64_t biggest = 0;
+  for (auto &t : forest.trees) biggest = std::max<int64_t>(biggest, (int64_t)t.NumNodes());
+  return biggest;
+}
+
+// Rows row-major in LDS, several lanes per row.
+LaunchPlan ChooseTreeParallelPlan(const Forest &forest, int64_t batchSize, const GPUAutoScheduleOptions *ov,
+                                  const DeviceLimits &limits) {
+  LaunchPlan plan;
+  plan.kernel = LaunchPlan::Kernel::kTreeParallel;
+  plan.interleave = 1;
+  if (ov && ov->treeWalkInterleaveFactor > 0)
+    plan.interleave = std::min(kMaxInterleave, FloorPow2(ov->treeWalkInterleaveFactor));
+  const int64_t rowBytes = (int64_t)(forest.numFeatures + 1) * 4;
+  const int64_t need = (BiggestTreeNodes(forest) + 2) * kNodeBytes;
+  if (need > 65536) throw Error("a tree does not fit one LDS tree group");
+  int64_t group = std::max<int64_t>(need, 24 * 1024);
+  const int64_t reserve = 4096; // reduction scratch and class sums
+  if (rowBytes + group + reserve > limits.ldsBytesPerBlock) group = need;
+  if (rowBytes + group + reserve > limits.ldsBytesPerBlock)
+    throw Error("a row of " + std::to_string(forest.numFeatures) + " features does not fit LDS next to a tree group");
+  int64_t rows = FloorPow2((limits.ldsBytesPerBlock - group - reserve) / rowBytes);
+  rows = std::min<int64_t>(rows, 16);
+  if (ov && ov->numRowsPerTB > 0) rows = std::min<int64_t>(rows, FloorPow2(ov->numRowsPerTB));
+  if (batchSize > 0) rows = std::min<int64_t>(rows, FloorPow2(std::max<int64_t>(batchSize, 1) * 2 - 1));
+  plan.rowsPerBlock = (int32_t)std::max<int64_t>(rows, 1);
+  plan.treeLanes = std::max(1, 256 / plan.rowsPerBlock);
+  // narrow rows leave LDS for bigger groups
+  const int64_t rowTile = rowBytes * plan.rowsPerBlock;
+  group = std::max<int64_t>(group, std::min<int64_t>(65536, (limits.ldsBytesPerBlock / 2 - rowTile - reserve)));
+  plan.groupBytes = (int32_t)(std::min<int64_t>(group, 65536) & ~15);
+
+  const int64_t rowBlocks = std::max<int64_t>(1, (batchSize + plan.rowsPerBlock - 1) / plan.rowsPerBlock);
+  const int64_t totalBytes = (int64_t)forest.NumNodes() * kNodeBytes;
+  int64_t groups = std::max<int64_t>(1, (totalBytes + plan.groupBytes - 1) / plan.groupBytes);
+  int64_t slices = 1;
+  const int64_t wantBlocks = 2LL * limits.computeUnits;
+  if (rowBlocks < wantBlocks) slices = (wantBlocks + rowBlocks - 1) / rowBlocks;
+  if (ov && ov->numTreeThreads > 0) slices = ov->numTreeThreads;
+  slices = std::min<int64_t>(slices, std::max<int64_t>(1, totalBytes / 8192)); // at least 8 KB of trees per slice
+  if (slices > groups) {
+    int64_t perSlice = std::max<int64_t>((totalBytes + slices - 1) / slices + 2048, need);
+    plan.groupBytes = (int32_t)(std::min<int64_t>(perSlice, 65536) & ~15);
+  }
+  plan.treeSlices = (int32_t)std::max<int64_t>(1, slices);
+  return plan;
+}
+
+} // namespace
+
 LaunchPlan ChoosePlan(const Forest &forest, int64_t batchSize, const GPUAutoScheduleOptions *ov,
                       const DeviceLimits &limits) {
+  bool fitsTransposed = false;
+  {
+    bool words = false;
+    fitsTransposed = RowTileFits(forest.numFeatures, 64, limits.ldsBytesPerBlock, &words);
+  }
+  if (!fitsTransposed || (batchSize > 0 && batchSize <= 128))
+    return ChooseTreeParallelPlan(forest, batchSize, ov, limits);
+
   LaunchPlan plan;
   plan.kernel = LaunchPlan::Kernel::kRowParallelLds;
 
@@ -82,6 +143,18 @@ std::vector<LaunchPlan> CandidatePlans(const Forest &forest, int64_t batchSize, 
   std::vector<LaunchPlan> out;
   LaunchPlan base = ChoosePlan(forest, batchSize, nullptr, limits);
   out.push_back(base);
+  if (base.kernel == LaunchPlan::Kernel::kTreeParallel) {
+    for (int32_t lanes : {base.treeLanes / 2, base.treeLanes * 2})
+      for (int32_t k : {1, 2}) {
+        LaunchPlan p = base;
+        p.treeLanes = lanes;
+        p.interleave = k;
+        if (lanes < 1 || p.ThreadsPerBlock() > 1024 || p.ThreadsPerBlock() % 64 != 0) continue;
+        if (lanes < 64 && 64 % lanes != 0) continue;
+        out.push_back(p);
+      }
+    return out;
+  }
   for (int32_t rb : {64, 128, 256, 512})
     for (int32_t k : {2, 4, 8})
       for (int blocksPerCu : {1, 2, 3}) {

@@ -59,6 +59,7 @@ SIGNATURES = {
                                   ctypes.POINTER(ctypes.c_double)]),
     "tbmi_autotune": (c_i32, [c_ip, c_vp, c_i64, ctypes.POINTER(ctypes.c_double)]),
     "tbmi_set_plan": (c_i32, [c_ip, c_i32, c_i32, c_i32, c_i32]),
+    "tbmi_set_tree_parallel_plan": (c_i32, [c_ip, c_i32, c_i32, c_i32, c_i32, c_i32]),
     "tbmi_describe_plan": (c_i32, [c_ip, c_cp, c_i32]),
     "tbmi_num_trees": (c_i32, [c_ip]),
     "tbmi_num_classes": (c_i32, [c_ip]),
