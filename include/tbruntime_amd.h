@@ -126,9 +126,11 @@ TBAMD_EXPORT int32_t tbmi_time_kernels(intptr_t runner, const float *deviceInput
                                        int64_t rows, int32_t runs, double *walkMs, double *finalizeMs);
 /* Timed search over launch plans on the given rows; keeps the fastest plan. */
 TBAMD_EXPORT int32_t tbmi_autotune(intptr_t runner, const float *deviceInputs, int64_t rows, double *bestMs);
-/* Pins a launch plan (values <= 0 keep the current one). */
-TBAMD_EXPORT int32_t tbmi_set_plan(intptr_t runner, int32_t rowsPerBlock, int32_t interleave, int32_t groupBytes,
-                                   int32_t treeSlices);
+/* Pins the row-parallel kernel: rowsPerBlock rows per block, treeThreads lanes per row (in different
+ * waves), interleave trees walked at once per lane, groupBytes of LDS per tree group, treeSlices blocks
+ * per row block (values <= 0 keep the current choice; treeThreads <= 0 means 1). */
+TBAMD_EXPORT int32_t tbmi_set_plan(intptr_t runner, int32_t rowsPerBlock, int32_t treeThreads, int32_t interleave,
+                                   int32_t groupBytes, int32_t treeSlices);
 /* Pins the tree-parallel kernel: rowsPerBlock rows per block, treeLanes lanes per row. */
 TBAMD_EXPORT int32_t tbmi_set_tree_parallel_plan(intptr_t runner, int32_t rowsPerBlock, int32_t treeLanes,
                                                  int32_t interleave, int32_t groupBytes, int32_t treeSlices);

@@ -195,14 +195,18 @@ def test_full_size_properties(synth_model, k):
 # --------------------------------------------------------------------------
 # launch plans, edge cases, API behaviour
 # --------------------------------------------------------------------------
-@pytest.mark.parametrize("plan", [(64, 1, 16384, 1), (128, 2, 32768, 3), (256, 8, 65536, 1), (512, 4, 49152, 5),
-                                  (256, 4, 8192, 40)])
-def test_launch_plans_agree(synth_model, plan):
-    forest = model_io.load_xgboost_json(synth_model(2))
-    x = synth.CONFIGS[2].batch_rows(3001, seed_offset=9)
-    runner = make_runner(synth_model(2), 3001)
+@pytest.mark.parametrize("plan", [(64, 1, 1, 16384, 1), (128, 1, 2, 32768, 3), (256, 1, 8, 65536, 1), (512, 1, 4, 49152, 5),
+                                  (256, 1, 4, 8192, 40), (256, 4, 4, 65536, 1), (128, 8, 2, 40960, 2), (64, 3, 1, 16384, 1),
+                                  (512, 2, 8, 32768, 1)])
+@pytest.mark.parametrize("k", [2, 3])
+def test_launch_plans_agree(synth_model, k, plan):
+    if k == 3 and plan[0] == 512:
+        pytest.skip("54 features x 512 rows exceed the LDS row tile")
+    forest = model_io.load_xgboost_json(synth_model(k))
+    x = synth.CONFIGS[k].batch_rows(3001, seed_offset=9)
+    runner = make_runner(synth_model(k), 3001)
     runner.set_plan(*plan)
-    assert "kernel=rows_lds rowsPerBlock=%d treeLanes=1 interleave=%d" % plan[:2] in runner.describe_plan()
+    assert "kernel=rows_lds rowsPerBlock=%d treeThreads=%d treeLanes=1 interleave=%d" % plan[:3] in runner.describe_plan()
     check_against_oracle(runner, forest, x)
 
 
@@ -214,7 +218,7 @@ def test_tree_parallel_plans_agree(synth_model, k, plan):
     x = synth.CONFIGS[k].batch_rows(203, seed_offset=3)
     runner = make_runner(synth_model(k), 203)
     runner.set_tree_parallel_plan(*plan)
-    assert "kernel=tree_parallel rowsPerBlock=%d treeLanes=%d" % plan[:2] in runner.describe_plan()
+    assert "kernel=tree_parallel rowsPerBlock=%d treeThreads=1 treeLanes=%d" % plan[:2] in runner.describe_plan()
     check_against_oracle(runner, forest, x)
 
 
@@ -294,3 +298,26 @@ def test_kernel_time_shim(synth_model):
     out = torch.zeros(1024, dtype=torch.float32, device="cuda")
     walk_ms, fin_ms = runner.time_kernels(dx.data_ptr(), out.data_ptr(), 1024, 5)
     assert 0 < walk_ms < 50 and fin_ms >= 0
+
+
+@pytest.mark.parametrize("rows", [1, 3, 63, 64, 65, 255, 257, 1000])
+@pytest.mark.parametrize("features,offset", [(3, 0), (5, 1), (28, 0), (28, 3), (33, 2)])
+def test_row_staging_alignment_and_ragged_tails(tmp_path, rows, features, offset):
+    """Inputs that start off a 16-byte boundary, odd feature counts and batches that end inside a block."""
+    rng = np.random.Generator(np.random.PCG64(features * 1000 + rows))
+    trees = [synth._grow_tree(rng, 5, lambda d, s: 0.9, lambda: (rng.integers(0, features), rng.normal()),
+                              lambda: rng.normal()) for _ in range(20)]
+    path = tmp_path / "m.json"
+    synth.write_xgboost_json(path, trees, features)
+    forest = model_io.load_xgboost_json(path)
+    x = rng.normal(size=(rows, features)).astype(np.float32)
+    expected, _ = cpu_oracle.predict(forest, x)
+    flat = torch.zeros(rows * features + 8, dtype=torch.float32, device="cuda")
+    flat[offset:offset + rows * features] = torch.from_numpy(x.reshape(-1)).cuda()
+    out = torch.zeros(rows, dtype=torch.float32, device="cuda")
+    for setup in (lambda r: None, lambda r: r.set_plan(64, 2, 2, 16384, 1), lambda r: r.set_tree_parallel_plan(4, 16, 1, 16384, 1)):
+        runner = make_runner(path, rows)
+        setup(runner)
+        out.fill_(float("nan"))
+        runner.run_device(flat.data_ptr() + 4 * offset, out.data_ptr(), rows)
+        np.testing.assert_allclose(out.cpu().numpy(), expected, rtol=RTOL_SUM, atol=0)

@@ -87,7 +87,7 @@ def test_synthetic_models_load_and_pack(lib, synth_model, k):
     h = load_forest(lib, path)
     assert_same_forest(lib, h, model_io.load_xgboost_json(path))
     stats = (ctypes.c_int64 * 5)()
-    for rows_per_block, interleave, group_bytes in [(256, 4, 49152), (128, 8, 65536), (64, 1, 32768), (256, 2, 16384)]:
+    for rows_per_block, interleave, group_bytes in [(256, 4, 49152), (128, 8, 32768), (64, 1, 16384), (256, 2, 16384)]:
         assert lib.tbmi_pack_roundtrip(h, rows_per_block, interleave, group_bytes, stats) == 0, last_error()
         assert stats[3] <= 160 * 1024
     lib.tbmi_delete_forest(h)
@@ -120,7 +120,7 @@ def test_onnx_comparison_modes_and_encodings(lib, tmp_path, mode, packed):
 def test_pack_rejects_plans_that_cannot_hold_the_model(lib, synth_model):
     h = load_forest(lib, synth_model(5))
     stats = (ctypes.c_int64 * 5)()
-    assert lib.tbmi_pack_roundtrip(h, 256, 4, 1024, stats) == -1      # deepest tree > one group
+    assert lib.tbmi_pack_roundtrip(h, 256, 4, 2048, stats) == -1      # deepest tree > one group
     assert "does not fit" in last_error()
     assert lib.tbmi_pack_roundtrip(h, 256, 3, 65536, stats) == -1     # interleave not a power of two
     assert lib.tbmi_pack_roundtrip(h, 1024, 4, 65536, stats) == -1    # 16-bit feature offsets overflow

@@ -38,10 +38,10 @@ struct DeviceNode {
 
 struct alignas(32) DeviceBundle {
   uint16_t root[kMaxInterleave]; // byte address of each tree's root inside the group
-  uint16_t depth;                // walk steps that bring every row to a leaf
-  uint16_t classId;
+  uint32_t depth;                // walk steps that bring every row to a leaf
+  uint32_t classId;              // (32-bit fields: the kernels fetch a bundle with scalar loads only)
   uint32_t firstSlot;            // index of root[0] in the slot->tree table
-  uint32_t reserved[2];
+  uint32_t reserved;
 };
 
 struct DeviceGroup {

@@ -17,7 +17,8 @@ struct WalkScalars {
   uint32_t groupRegionBytes = 0; // LDS bytes reserved for one tree group (multiple of 16)
   int32_t transform = 0;         // 0 identity, 1 sigmoid
   int32_t numTrees = 0;
-  int32_t rowsPerBlock = 0;      // tree-parallel kernel: rows per block
+  int32_t rowsPerBlock = 0;      // rows per block (both kernels)
+  int32_t treeThreads = 1;       // row-parallel kernel: lanes (in different waves) that share a row
   int32_t treeLanes = 1;         // tree-parallel kernel: lanes per row (power of two)
   double initialValue = 0.0;
 };
@@ -29,7 +30,7 @@ struct WalkParams {
   const DeviceBundle *bundles = nullptr;
   const DeviceGroup *groups = nullptr;
   float *out = nullptr;           // used when the epilogue is fused (1 slice, no classes)
-  double *partial = nullptr;      // [slices][rows][max(1, classes)] otherwise
+  double *partial = nullptr;      // [partials][rows][max(1, classes)] otherwise
   // leaf-id dump (parity checks only)
   int32_t *leafIds = nullptr;     // [rows][numTrees]
   const int32_t *nodeOrigin = nullptr;
@@ -40,7 +41,7 @@ struct FinalizeParams {
   const double *partial = nullptr; // [slices][rows][max(1, classes)]
   int64_t rows = 0;
   int32_t numClasses = 0;
-  int32_t treeSlices = 1;
+  int32_t treeSlices = 1;      // number of partial sums per (row, class)
   double initialValue = 0.0;
   int32_t transform = 0;
   float *out = nullptr;        // regression / binary prediction, may be null for multiclass
@@ -49,10 +50,10 @@ struct FinalizeParams {
   float *probabilities = nullptr; // optional [rows][classes] softmax
 };
 
-// Row-parallel walk over LDS-staged tree groups.  `interleave` in {1,2,4,8};
-// `featureOffsetInWords` selects how node feature offsets are scaled.
-hipError_t LaunchWalkRowsLds(const WalkParams &p, int rowsPerBlock, int interleave, bool featureOffsetInWords,
-                             size_t ldsBytes, hipStream_t stream);
+// Row-parallel walk over LDS-staged tree groups: block = s.rowsPerBlock * s.treeThreads lanes.
+// `interleave` in {1,2,4,8}; `featureOffsetInWords` selects how node feature offsets are scaled.
+hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, bool featureOffsetInWords, size_t ldsBytes,
+                             hipStream_t stream);
 // Tree-parallel walk: s.rowsPerBlock rows per block (row-major in LDS),
 // s.treeLanes lanes per row; block = rowsPerBlock * treeLanes lanes.
 hipError_t LaunchWalkTreeParallel(const WalkParams &p, int interleave, size_t ldsBytes, hipStream_t stream);

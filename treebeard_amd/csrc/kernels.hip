@@ -20,21 +20,92 @@ __device__ __forceinline__ float AsFloat(uint32_t u) { return __uint_as_float(u)
 // which the compiler places at LDS address 0, so an offset into the dynamic
 // array is the address itself and no base has to be added per access.
 typedef uint32_t U32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
 typedef const __attribute__((address_space(3))) U32x2 *LdsNodePtr;
 typedef const __attribute__((address_space(3))) float *LdsFloatPtr;
 __device__ __forceinline__ U32x2 LdsLoadNode(uint32_t address) { return *(LdsNodePtr)(uintptr_t)address; }
 __device__ __forceinline__ float LdsLoadFloat(uint32_t address) { return *(LdsFloatPtr)(uintptr_t)address; }
 
+
+// Copies the block's rows (contiguous, row-major in global memory) into the LDS tile.
+// kTransposed: tile[f * R + r] (row-parallel kernel), else tile[r * rowWords + f].
+// Loads are 16-byte wide, issued kStageUnroll at a time per lane and unconditional (index
+// clamped into the live part of the batch) so that they overlap; rows past the end of the
+// batch read as 0 and nothing outside the batch is touched.
+constexpr int kStageUnroll = 8;
+
+template <bool kTransposed>
+__device__ __forceinline__ void StageRows(const float *__restrict__ src, int valid, int R, int F, int rowWords,
+                                          float *tile, int tid, int threads) {
+  const int total = R * F;
+  const int live = valid * F;
+  const bool aligned = (reinterpret_cast<uintptr_t>(src) & 15u) == 0;
+  const int vecs = aligned ? total >> 2 : 0;    // 16-byte pieces handled by the vector path
+  const int liveVecs = aligned ? live >> 2 : 0; // pieces that lie entirely inside the batch
+  const float invF = 1.0f / (float)F;
+  typedef float F32x4 __attribute__((ext_vector_type(4)));
+  const F32x4 *src4 = reinterpret_cast<const F32x4 *>(src);
+  for (int base = 0; base < vecs; base += threads * kStageUnroll) {
+    F32x4 v[kStageUnroll];
+#pragma unroll
+    for (int u = 0; u < kStageUnroll; ++u) {
+      const int idx = base + u * threads + tid;
+      const int clamped = idx < liveVecs ? idx : (liveVecs > 0 ? liveVecs - 1 : 0);
+      v[u] = liveVecs > 0 ? src4[clamped] : F32x4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int u = 0; u < kStageUnroll; ++u) {
+      const int idx = base + u * threads + tid;
+      if (idx >= vecs) continue;
+      const int e0 = idx << 2;
+      int r = (int)((float)e0 * invF);
+      if (r * F > e0) --r;
+      if ((r + 1) * F <= e0) ++r;
+      int f = e0 - r * F;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int e = e0 + j;
+        // elements of the one partially live piece are left to the scalar tail below
+        if (idx < liveVecs || e >= live) {
+          const float value = idx < liveVecs ? v[u][j] : 0.0f;
+          if (kTransposed) tile[f * R + r] = value;
+          else tile[r * rowWords + f] = value;
+        }
+        if (++f == F) { f = 0; ++r; }
+      }
+    }
+  }
+  // scalar: the live elements of the partially live piece, which the vector path skipped ...
+  const int skippedEnd = live < (vecs << 2) ? live : (vecs << 2);
+  for (int e = (liveVecs << 2) + tid; e < skippedEnd; e += threads) {
+    const int r = e / F;
+    const int f = e - r * F;
+    if (kTransposed) tile[f * R + r] = src[e];
+    else tile[r * rowWords + f] = src[e];
+  }
+  // ... and whatever lies behind the last whole 16-byte piece (everything, for unaligned input)
+  for (int e = (vecs << 2) + tid; e < total; e += threads) {
+    const int r = e / F;
+    const int f = e - r * F;
+    const float value = e < live ? src[e] : 0.0f;
+    if (kTransposed) tile[f * R + r] = value;
+    else tile[r * rowWords + f] = value;
+  }
+}
+
 // ---------------------------------------------------------------------------
-// Row-parallel walk.  One lane owns one row of the block; the block's rows sit
-// transposed in LDS (feature-major) so that lane i always reads bank i%32 no
-// matter which feature its node tests.  Trees are streamed through LDS one
-// group at a time and walked K at a time in lock step: all lanes take `depth`
-// steps, leaves hold the walk in place (see device_model.h), so the loop body
-// has no leaf test and no divergence.  The per-row sum is kept in double and
-// trees are added in packed order.
+// Row-parallel walk.  The block owns `rowsPerBlock` rows, kept transposed in
+// LDS (feature-major) so that lane i always reads bank i%64 no matter which
+// feature its node tests.  Trees are streamed through LDS one group at a time;
+// the next group is fetched into registers while the current one is walked.
+// A lane walks K trees at a time in lock step: all lanes take `depth` steps and
+// leaves hold the walk in place (see device_model.h), so the loop body has no
+// leaf test and no divergence.  `treeThreads` lanes (in different waves) share
+// one row and split each group's bundles between them, which buys occupancy
+// without growing the row tile; their sums meet in an LDS cross-wave pass.
+// Sums are kept in double; trees are added in packed order.
 // ---------------------------------------------------------------------------
-template <int K, bool kOffsetsInWords, bool kDump>
+template <int K, int PF, bool kOffsetsInWords, bool kDump>
 __global__ void __launch_bounds__(1024)
 WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16,
                   const DeviceBundle *__restrict__ bundles, const DeviceGroup *__restrict__ groups,
@@ -45,101 +116,152 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
   // address 0 so that node pointers are LDS addresses as stored.
   extern __shared__ __align__(16) unsigned char lds[];
   const int tid = threadIdx.x;
-  const int RB = blockDim.x;
+  const int threads = blockDim.x;
+  const int RB = s.rowsPerBlock;
+  const int TT = s.treeThreads;
+  const int lane = tid & (RB - 1);
+  // uniform inside a wave (RB is a multiple of 64); readfirstlane tells the compiler so
+  const int tt = __builtin_amdgcn_readfirstlane(tid / RB);
   const int F = s.numFeatures;
   const int64_t row0 = (int64_t)blockIdx.x * RB;
   const int64_t remaining = s.rows - row0;
   const int valid = remaining < RB ? (int)remaining : RB;
 
-  unsigned char *group = lds;
   float *rowTile = reinterpret_cast<float *>(lds + s.groupRegionBytes);
 
-  // Stage the block's rows: coalesced reads of the contiguous row-major tile,
-  // transposed writes.  Rows past the end of the batch read as 0.
-  {
-    const float *src = x + row0 * F;
-    const int total = RB * F;
-    const int live = valid * F;
-    for (int e = tid; e < total; e += RB) {
-      const int r = e / F;
-      const int f = e - r * F;
-      rowTile[f * RB + r] = e < live ? src[e] : 0.0f;
-    }
-    rowTile[F * RB + tid] = -INFINITY; // pad feature: keeps leaves in place
-  }
-  const uint32_t column = s.groupRegionBytes + (uint32_t)tid * 4u; // LDS address of this row's feature 0
+  // Stage the block's rows: coalesced reads of the contiguous row-major tile, transposed writes.
+  StageRows<true>(x + row0 * F, valid, RB, F, 0, rowTile, tid, threads);
+  for (int i = tid; i < RB; i += threads) rowTile[F * RB + i] = -INFINITY; // pad feature: keeps leaves in place
+  const uint32_t column = s.groupRegionBytes + (uint32_t)lane * 4u; // LDS address of this row's feature 0
 
   const int slice = blockIdx.y;
   const int gBegin = (int)(((int64_t)s.numGroups * slice) / s.treeSlices);
   const int gEnd = (int)(((int64_t)s.numGroups * (slice + 1)) / s.treeSlices);
   const int C = s.numClasses;
-  const int64_t row = row0 + tid;
+  const int64_t row = row0 + lane;
   double *partialRow = partial ? partial + ((int64_t)slice * s.rows + row) * (C > 0 ? C : 1) : nullptr;
+  // LDS cross-wave pass: the tree threads of a row leave their sums here and tree thread 0 adds
+  // them in thread order.  Classifiers meet at class boundaries, while a tree group is live, so
+  // their meeting area sits behind the row tile; otherwise the (then idle) group region is used.
+  double *meet = reinterpret_cast<double *>(C > 0 ? lds + s.groupRegionBytes + (uint32_t)(F + 1) * RB * 4u : lds);
 
   double acc = 0.0;
   int curClass = 0;
+
+  // Register double buffer for the next tree group.  Loads are unconditional
+  // (index clamped) so that they stay in flight across the walk.
+  U32x4 fetched[PF];
+#define TBAMD_PREFETCH_GROUP(G)                                                                                        \
+  {                                                                                                                    \
+    const DeviceGroup nextGrp = groups[(G)];                                                                           \
+    const U32x4 *src = reinterpret_cast<const U32x4 *>(nodes16) + (nextGrp.nodeBegin >> 1);                            \
+    const int last = (int)(nextGrp.nodeCount >> 1) - 1;                                                                \
+    _Pragma("unroll") for (int i = 0; i < PF; ++i) {                                                                   \
+      const int idx = tid + i * threads;                                                                               \
+      fetched[i] = src[idx < last ? idx : last];                                                                       \
+    }                                                                                                                  \
+  }
+  // Ends class `curClass`: the row's tree threads meet in LDS and thread 0 stores the class sum.
+  // Uniform across the block (class boundaries are bundle positions), so the barriers are safe.
+#define TBAMD_FLUSH_CLASS(UPTO)                                                                                        \
+  {                                                                                                                    \
+    if (TT > 1) {                                                                                                      \
+      __syncthreads();                                                                                                 \
+      meet[tid] = acc;                                                                                                 \
+      __syncthreads();                                                                                                 \
+      if (tt == 0) {                                                                                                   \
+        acc = 0.0;                                                                                                     \
+        for (int t = 0; t < TT; ++t) acc += meet[t * RB + lane];                                                       \
+      }                                                                                                                \
+    }                                                                                                                  \
+    if (tt == 0 && lane < valid) {                                                                                     \
+      partialRow[curClass] = acc;                                                                                      \
+      for (int c = curClass + 1; c < (UPTO); ++c) partialRow[c] = 0.0;                                                 \
+    }                                                                                                                  \
+    acc = 0.0;                                                                                                         \
+  }
+  if (gBegin < gEnd) TBAMD_PREFETCH_GROUP(gBegin)
 
   for (int g = gBegin; g < gEnd; ++g) {
     const DeviceGroup grp = groups[g];
     __syncthreads(); // rows staged / previous group no longer read
     {
-      const uint4 *src = nodes16 + (grp.nodeBegin >> 1);
-      uint4 *dst = reinterpret_cast<uint4 *>(group);
+      U32x4 *dst = reinterpret_cast<U32x4 *>(lds);
       const int pieces = (int)(grp.nodeCount >> 1);
-      for (int i = tid; i < pieces; i += RB) dst[i] = src[i];
+#pragma unroll
+      for (int i = 0; i < PF; ++i) {
+        const int idx = tid + i * threads;
+        if (idx < pieces) dst[idx] = fetched[i];
+      }
     }
     __syncthreads();
+    if (g + 1 < gEnd) TBAMD_PREFETCH_GROUP(g + 1) // in flight while this group is walked
 
-    for (uint32_t b = 0; b < grp.bundleCount; ++b) {
-      const DeviceBundle bd = bundles[grp.bundleBegin + b];
+    // Bundles are sorted by class; a segment is a run of bundles of one class.
+    uint32_t b0 = 0;
+    while (b0 < grp.bundleCount) {
+      uint32_t b1 = grp.bundleCount;
       if (C > 0) {
-        const int cls = bd.classId;
+        const int cls = (int)bundles[grp.bundleBegin + b0].classId;
         if (cls != curClass) { // classes arrive in ascending order
-          if (tid < valid) {
-            partialRow[curClass] = acc;
-            for (int c = curClass + 1; c < cls; ++c) partialRow[c] = 0.0;
-          }
-          acc = 0.0;
+          TBAMD_FLUSH_CLASS(cls)
           curClass = cls;
         }
+        b1 = b0 + 1;
+        while (b1 < grp.bundleCount && (int)bundles[grp.bundleBegin + b1].classId == cls) ++b1;
       }
-      uint32_t addr[K];
+      for (uint32_t b = b0 + tt; b < b1; b += TT) {
+        const DeviceBundle bd = bundles[grp.bundleBegin + b];
+        uint32_t addr[K];
 #pragma unroll
-      for (int k = 0; k < K; ++k) addr[k] = bd.root[k];
-      const int depth = bd.depth;
-      for (int d = 0; d < depth; ++d) {
-#pragma unroll
-        for (int k = 0; k < K; ++k) {
-          const U32x2 node = LdsLoadNode(addr[k]);
-          const uint32_t off = kOffsetsInWords ? (node.y & 0xFFFFu) << 2 : (node.y & 0xFFFFu);
-          const float xv = LdsLoadFloat(column + off);
-          addr[k] = (node.y >> 16) + (xv < AsFloat(node.x) ? 0u : kNodeBytes);
-        }
-      }
-#pragma unroll
-      for (int k = 0; k < K; ++k) acc += (double)LdsLoadFloat(addr[k]);
-      if (kDump) {
-        if (tid < valid) {
+        for (int k = 0; k < K; ++k) addr[k] = bd.root[k];
+        const int depth = (int)bd.depth;
+        for (int d = 0; d < depth; ++d) {
 #pragma unroll
           for (int k = 0; k < K; ++k) {
-            const int tree = slotTree[bd.firstSlot + k];
-            if (tree >= 0) leafIds[row * s.numTrees + tree] = nodeOrigin[grp.nodeBegin + addr[k] / kNodeBytes];
+            const U32x2 node = LdsLoadNode(addr[k]);
+            const uint32_t off = kOffsetsInWords ? (node.y & 0xFFFFu) << 2 : (node.y & 0xFFFFu);
+            const float xv = LdsLoadFloat(column + off);
+            addr[k] = (node.y >> 16) + (xv < AsFloat(node.x) ? 0u : kNodeBytes);
+          }
+        }
+#pragma unroll
+        for (int k = 0; k < K; ++k) acc += (double)LdsLoadFloat(addr[k]);
+        if (kDump) {
+          if (lane < valid) {
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+              const int tree = slotTree[bd.firstSlot + k];
+              if (tree >= 0) leafIds[row * s.numTrees + tree] = nodeOrigin[grp.nodeBegin + addr[k] / kNodeBytes];
+            }
           }
         }
       }
+      b0 = b1;
     }
   }
 
-  if (tid >= valid) return;
   if (C > 0) {
-    partialRow[curClass] = acc;
-    for (int c = curClass + 1; c < C; ++c) partialRow[c] = 0.0;
-  } else if (partial) {
+    TBAMD_FLUSH_CLASS(C)
+    return;
+  }
+  if (TT > 1) {
+    __syncthreads();
+    meet[tid] = acc;
+    __syncthreads();
+    if (tt != 0) return;
+    acc = 0.0;
+    for (int t = 0; t < TT; ++t) acc += meet[t * RB + lane];
+  }
+  if (lane >= valid) return;
+  if (partial) {
     partialRow[0] = acc;
   } else {
     const double margin = s.initialValue + acc;
     out[row] = (float)(s.transform == 1 ? 1.0 / (1.0 + exp(-margin)) : margin);
   }
+#undef TBAMD_FLUSH_CLASS
+#undef TBAMD_PREFETCH_GROUP
 }
 
 // ---------------------------------------------------------------------------
@@ -160,7 +282,7 @@ __device__ __forceinline__ double ShuffleXor(double v, int mask) {
   return __hiloint2double(hi, lo);
 }
 
-template <int K, bool kDump>
+template <int K, int PF, bool kDump>
 __global__ void __launch_bounds__(1024)
 WalkTreeParallelKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16,
                        const DeviceBundle *__restrict__ bundles, const DeviceGroup *__restrict__ groups,
@@ -188,18 +310,9 @@ WalkTreeParallelKernel(const float *__restrict__ x, const uint4 *__restrict__ no
   double *waveScratch = reinterpret_cast<double *>(lds + scratchOffset);
   double *classSums = waveScratch + (threads + 63) / 64;
 
-  {
-    const float *src = x + row0 * F;
-    const int total = R * F;
-    const int live = valid * F;
-    for (int e = tid; e < total; e += threads) {
-      const int rr = e / F;
-      const int f = e - rr * F;
-      rowsLds[rr * rowWords + f] = e < live ? src[e] : 0.0f;
-    }
-    for (int rr = tid; rr < R; rr += threads) rowsLds[rr * rowWords + F] = -INFINITY;
-    for (int i = tid; i < R * Cn; i += threads) classSums[i] = 0.0;
-  }
+  StageRows<false>(x + row0 * F, valid, R, F, rowWords, rowsLds, tid, threads);
+  for (int rr = tid; rr < R; rr += threads) rowsLds[rr * rowWords + F] = -INFINITY;
+  for (int i = tid; i < R * Cn; i += threads) classSums[i] = 0.0;
   const uint32_t rowBase = s.groupRegionBytes + (uint32_t)r * rowWords * 4u;
 
   const int slice = blockIdx.y;
@@ -207,16 +320,34 @@ WalkTreeParallelKernel(const float *__restrict__ x, const uint4 *__restrict__ no
   const int gEnd = (int)(((int64_t)s.numGroups * (slice + 1)) / s.treeSlices);
   const int64_t row = row0 + r;
 
+  // Register double buffer for the next tree group (loads stay in flight across the walk).
+  U32x4 fetched[PF];
+#define TBAMD_PREFETCH_GROUP(G)                                                                                        \
+  {                                                                                                                    \
+    const DeviceGroup nextGrp = groups[(G)];                                                                           \
+    const U32x4 *src = reinterpret_cast<const U32x4 *>(nodes16) + (nextGrp.nodeBegin >> 1);                            \
+    const int last = (int)(nextGrp.nodeCount >> 1) - 1;                                                                \
+    _Pragma("unroll") for (int i = 0; i < PF; ++i) {                                                                   \
+      const int idx = tid + i * threads;                                                                               \
+      fetched[i] = src[idx < last ? idx : last];                                                                       \
+    }                                                                                                                  \
+  }
+  if (gBegin < gEnd) TBAMD_PREFETCH_GROUP(gBegin)
+
   for (int g = gBegin; g < gEnd; ++g) {
     const DeviceGroup grp = groups[g];
     __syncthreads();
     {
-      const uint4 *src = nodes16 + (grp.nodeBegin >> 1);
-      uint4 *dst = reinterpret_cast<uint4 *>(lds);
+      U32x4 *dst = reinterpret_cast<U32x4 *>(lds);
       const int pieces = (int)(grp.nodeCount >> 1);
-      for (int i = tid; i < pieces; i += threads) dst[i] = src[i];
+#pragma unroll
+      for (int i = 0; i < PF; ++i) {
+        const int idx = tid + i * threads;
+        if (idx < pieces) dst[idx] = fetched[i];
+      }
     }
     __syncthreads();
+    if (g + 1 < gEnd) TBAMD_PREFETCH_GROUP(g + 1)
 
     // bundles are sorted by class: handle one class segment at a time
     uint32_t b0 = 0;
@@ -278,6 +409,7 @@ WalkTreeParallelKernel(const float *__restrict__ x, const uint4 *__restrict__ no
     const double margin = s.initialValue + classSums[r];
     out[row] = (float)(s.transform == 1 ? 1.0 / (1.0 + exp(-margin)) : margin);
   }
+#undef TBAMD_PREFETCH_GROUP
 }
 
 // ---------------------------------------------------------------------------
@@ -326,66 +458,86 @@ __global__ void __launch_bounds__(256) FinalizeKernel(const FinalizeParams p) {
   }
 }
 
-template <int K, bool W>
-hipError_t LaunchWalkK(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
+template <int K, int PF, bool W>
+hipError_t LaunchWalkKP(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
   if (p.leafIds) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&WalkRowsLdsKernel<K, W, true>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&WalkRowsLdsKernel<K, PF, W, true>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
     if (e != hipSuccess) return e;
-    WalkRowsLdsKernel<K, W, true><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out, p.partial,
-                                                                     p.leafIds, p.nodeOrigin, p.slotTree);
+    WalkRowsLdsKernel<K, PF, W, true><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out,
+                                                                         p.partial, p.leafIds, p.nodeOrigin, p.slotTree);
   } else {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&WalkRowsLdsKernel<K, W, false>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&WalkRowsLdsKernel<K, PF, W, false>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
     if (e != hipSuccess) return e;
-    WalkRowsLdsKernel<K, W, false><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out,
-                                                                      p.partial, nullptr, nullptr, nullptr);
+    WalkRowsLdsKernel<K, PF, W, false><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out,
+                                                                          p.partial, nullptr, nullptr, nullptr);
   }
   return hipGetLastError();
 }
 
+template <int K, bool W>
+hipError_t LaunchWalkK(const WalkParams &p, int prefetch, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
+  if (prefetch <= 4) return LaunchWalkKP<K, 4, W>(p, grid, block, ldsBytes, stream);
+  if (prefetch <= 8) return LaunchWalkKP<K, 8, W>(p, grid, block, ldsBytes, stream);
+  if (prefetch <= 16) return LaunchWalkKP<K, 16, W>(p, grid, block, ldsBytes, stream);
+  return hipErrorInvalidValue;
+}
+
 template <bool W>
-hipError_t LaunchWalkW(const WalkParams &p, int interleave, dim3 grid, dim3 block, size_t ldsBytes,
+hipError_t LaunchWalkW(const WalkParams &p, int interleave, int prefetch, dim3 grid, dim3 block, size_t ldsBytes,
                        hipStream_t stream) {
   switch (interleave) {
-  case 1: return LaunchWalkK<1, W>(p, grid, block, ldsBytes, stream);
-  case 2: return LaunchWalkK<2, W>(p, grid, block, ldsBytes, stream);
-  case 4: return LaunchWalkK<4, W>(p, grid, block, ldsBytes, stream);
-  case 8: return LaunchWalkK<8, W>(p, grid, block, ldsBytes, stream);
+  case 1: return LaunchWalkK<1, W>(p, prefetch, grid, block, ldsBytes, stream);
+  case 2: return LaunchWalkK<2, W>(p, prefetch, grid, block, ldsBytes, stream);
+  case 4: return LaunchWalkK<4, W>(p, prefetch, grid, block, ldsBytes, stream);
+  case 8: return LaunchWalkK<8, W>(p, prefetch, grid, block, ldsBytes, stream);
   default: return hipErrorInvalidValue;
   }
 }
 
 } // namespace
 
-hipError_t LaunchWalkRowsLds(const WalkParams &p, int rowsPerBlock, int interleave, bool featureOffsetInWords,
-                             size_t ldsBytes, hipStream_t stream) {
+hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, bool featureOffsetInWords, size_t ldsBytes,
+                             hipStream_t stream) {
   if (p.s.rows <= 0) return hipSuccess;
-  if (ldsBytes > 160 * 1024) return hipErrorInvalidValue;
-  const int64_t blocks = (p.s.rows + rowsPerBlock - 1) / rowsPerBlock;
+  const int RB = p.s.rowsPerBlock, TT = p.s.treeThreads;
+  if (ldsBytes > 160 * 1024 || RB < 64 || (RB & (RB - 1)) || TT < 1 || RB * TT > 1024) return hipErrorInvalidValue;
+  const int64_t blocks = (p.s.rows + RB - 1) / RB;
   if (blocks > 0x7FFFFFFF || p.s.treeSlices < 1 || p.s.treeSlices > 65535) return hipErrorInvalidValue;
-  dim3 grid((unsigned)blocks, (unsigned)p.s.treeSlices), block((unsigned)rowsPerBlock);
-  return featureOffsetInWords ? LaunchWalkW<true>(p, interleave, grid, block, ldsBytes, stream)
-                              : LaunchWalkW<false>(p, interleave, grid, block, ldsBytes, stream);
+  // registers that hold the next tree group while the current one is walked
+  const int prefetch = (int)((p.s.groupRegionBytes / 16 + RB * TT - 1) / (RB * TT));
+  dim3 grid((unsigned)blocks, (unsigned)p.s.treeSlices), block((unsigned)(RB * TT));
+  return featureOffsetInWords ? LaunchWalkW<true>(p, interleave, prefetch, grid, block, ldsBytes, stream)
+                              : LaunchWalkW<false>(p, interleave, prefetch, grid, block, ldsBytes, stream);
 }
 
 namespace {
-template <int K>
-hipError_t LaunchTreeParallelK(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
+template <int K, int PF>
+hipError_t LaunchTreeParallelKP(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
   if (p.leafIds) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&WalkTreeParallelKernel<K, true>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&WalkTreeParallelKernel<K, PF, true>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
     if (e != hipSuccess) return e;
-    WalkTreeParallelKernel<K, true><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out,
-                                                                      p.partial, p.leafIds, p.nodeOrigin, p.slotTree);
+    WalkTreeParallelKernel<K, PF, true><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out,
+                                                                          p.partial, p.leafIds, p.nodeOrigin, p.slotTree);
   } else {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&WalkTreeParallelKernel<K, false>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&WalkTreeParallelKernel<K, PF, false>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
     if (e != hipSuccess) return e;
-    WalkTreeParallelKernel<K, false><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out,
-                                                                       p.partial, nullptr, nullptr, nullptr);
+    WalkTreeParallelKernel<K, PF, false><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out,
+                                                                           p.partial, nullptr, nullptr, nullptr);
   }
   return hipGetLastError();
+}
+
+template <int K>
+hipError_t LaunchTreeParallelK(const WalkParams &p, int prefetch, dim3 grid, dim3 block, size_t ldsBytes,
+                               hipStream_t stream) {
+  if (prefetch <= 4) return LaunchTreeParallelKP<K, 4>(p, grid, block, ldsBytes, stream);
+  if (prefetch <= 8) return LaunchTreeParallelKP<K, 8>(p, grid, block, ldsBytes, stream);
+  if (prefetch <= 16) return LaunchTreeParallelKP<K, 16>(p, grid, block, ldsBytes, stream);
+  return hipErrorInvalidValue;
 }
 } // namespace
 
@@ -396,12 +548,13 @@ hipError_t LaunchWalkTreeParallel(const WalkParams &p, int interleave, size_t ld
   if (threads > 1024 || threads % 64 != 0) return hipErrorInvalidValue;
   const int64_t blocks = (p.s.rows + p.s.rowsPerBlock - 1) / p.s.rowsPerBlock;
   if (blocks > 0x7FFFFFFF || p.s.treeSlices < 1 || p.s.treeSlices > 65535) return hipErrorInvalidValue;
+  const int prefetch = (int)((p.s.groupRegionBytes / 16 + threads - 1) / threads);
   dim3 grid((unsigned)blocks, (unsigned)p.s.treeSlices), block((unsigned)threads);
   switch (interleave) {
-  case 1: return LaunchTreeParallelK<1>(p, grid, block, ldsBytes, stream);
-  case 2: return LaunchTreeParallelK<2>(p, grid, block, ldsBytes, stream);
-  case 4: return LaunchTreeParallelK<4>(p, grid, block, ldsBytes, stream);
-  case 8: return LaunchTreeParallelK<8>(p, grid, block, ldsBytes, stream);
+  case 1: return LaunchTreeParallelK<1>(p, prefetch, grid, block, ldsBytes, stream);
+  case 2: return LaunchTreeParallelK<2>(p, prefetch, grid, block, ldsBytes, stream);
+  case 4: return LaunchTreeParallelK<4>(p, prefetch, grid, block, ldsBytes, stream);
+  case 8: return LaunchTreeParallelK<8>(p, prefetch, grid, block, ldsBytes, stream);
   default: return hipErrorInvalidValue;
   }
 }

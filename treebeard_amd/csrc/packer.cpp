@@ -34,6 +34,8 @@ size_t PackedModel::LdsBytes() const {
     const size_t waves = (size_t)(plan.ThreadsPerBlock() + 63) / 64;
     bytes = (bytes + 7) & ~(size_t)7;
     bytes += waves * 8 + (size_t)plan.rowsPerBlock * (numClasses > 0 ? numClasses : 1) * 8;
+  } else if (plan.treeThreads > 1 && numClasses > 0) {
+    bytes += (size_t)plan.ThreadsPerBlock() * 8; // classifiers: cross-wave pass behind the row tile
   }
   return bytes;
 }
@@ -69,12 +71,16 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
   if (plan.kernel == LaunchPlan::Kernel::kRowParallelLds) {
     if (plan.rowsPerBlock < 64 || (plan.rowsPerBlock & (plan.rowsPerBlock - 1)) || plan.rowsPerBlock > 1024)
       throw Error("rowsPerBlock must be a power of two in [64, 1024]");
+    if (plan.treeThreads < 1 || plan.ThreadsPerBlock() > 1024)
+      throw Error("rowsPerBlock * treeThreads must not exceed 1024 lanes");
   } else {
     if (plan.treeLanes < 1 || (plan.treeLanes & (plan.treeLanes - 1)) || plan.rowsPerBlock < 1 ||
         plan.ThreadsPerBlock() > 1024 || plan.ThreadsPerBlock() % 64 != 0)
       throw Error("tree-parallel plan needs a power-of-two treeLanes and a block of 64..1024 lanes");
     if (plan.treeLanes < 64 && 64 % plan.treeLanes != 0) throw Error("treeLanes must divide 64");
   }
+  if (plan.groupBytes > 256 * plan.ThreadsPerBlock())
+    throw Error("groupBytes must not exceed 256 bytes per lane of the block (group prefetch registers)");
   if (plan.groupBytes < 1024 || plan.groupBytes > 65536) throw Error("groupBytes must be in [1024, 65536]");
 
   PackedModel pm;
@@ -128,6 +134,9 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
     // one spare node keeps room for the alignment pad
     auto freeNodes = [&]() { return groupCapacity - 1 - ((uint32_t)pm.nodes.size() - g.nodeBegin); };
     bool any = false;
+    struct Mark { size_t nodes, slots, next; };
+    std::vector<Mark> marks; // state before each bundle of this group
+    const size_t multiple = plan.kernel == LaunchPlan::Kernel::kRowParallelLds ? (size_t)plan.treeThreads : 1;
     while (next < order.size()) {
       // gather up to K consecutive trees of one class that still fit
       DeviceBundle b{};
@@ -145,7 +154,8 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
         ++count;
       }
       if (count == 0) break; // group full
-      b.classId = (uint16_t)cls;
+      marks.push_back(Mark{pm.nodes.size(), pm.slotTree.size(), next});
+      b.classId = (uint32_t)cls;
       b.firstSlot = (uint32_t)pm.slotTree.size();
       for (int k = 0; k < K; ++k) {
         if (k >= count) {
@@ -158,7 +168,7 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
         const LevelOrder lo = MakeLevelOrder(tree);
         const uint32_t base = (uint32_t)pm.nodes.size() - g.nodeBegin; // node index inside the group
         b.root[k] = (uint16_t)(base * kNodeBytes);
-        b.depth = std::max<uint16_t>(b.depth, (uint16_t)depth[t]);
+        b.depth = std::max<uint32_t>(b.depth, (uint32_t)depth[t]);
         pm.slotTree.push_back(t);
         for (size_t i = 0; i < lo.order.size(); ++i) {
           const int32_t n = lo.order[i];
@@ -179,6 +189,16 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
       pm.bundles.push_back(b);
       next += count;
       any = true;
+    }
+    // Tree threads take bundles round-robin: when more trees follow, end the group on a
+    // multiple of treeThreads bundles so that no thread idles through a last partial round.
+    if (next < order.size() && multiple > 1 && marks.size() > multiple && marks.size() % multiple != 0) {
+      const size_t keep = marks.size() - marks.size() % multiple;
+      pm.nodes.resize(marks[keep].nodes);
+      pm.nodeOrigin.resize(marks[keep].nodes);
+      pm.slotTree.resize(marks[keep].slots);
+      pm.bundles.resize(g.bundleBegin + keep);
+      next = marks[keep].next;
     }
     closeGroup();
     if (!any) throw Error("internal error: empty tree group");

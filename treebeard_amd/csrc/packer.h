@@ -20,14 +20,17 @@ namespace tbamd {
 struct LaunchPlan {
   enum class Kernel : int32_t { kRowParallelLds = 0, kTreeParallel = 1 };
   Kernel kernel = Kernel::kRowParallelLds;
-  int32_t rowsPerBlock = 256;   // row-parallel: = threads per block, power of two
+  int32_t rowsPerBlock = 256;   // row-parallel: rows (= lanes per tree thread) per block, power of two
+  int32_t treeThreads = 1;      // row-parallel: lanes in different waves that share a row; block = rowsPerBlock * treeThreads
   int32_t treeLanes = 1;        // tree-parallel: lanes per row, power of two; block = rowsPerBlock * treeLanes
   int32_t interleave = 4;       // K: trees walked concurrently by one lane (1, 2, 4, 8)
   int32_t groupBytes = 48 * 1024; // LDS bytes for one tree group's nodes (<= 65536)
   int32_t treeSlices = 1;       // grid.y: how many blocks share one row block's trees
   bool featureOffsetInWords = false;
 
-  int32_t ThreadsPerBlock() const { return kernel == Kernel::kTreeParallel ? rowsPerBlock * treeLanes : rowsPerBlock; }
+  int32_t ThreadsPerBlock() const {
+    return kernel == Kernel::kTreeParallel ? rowsPerBlock * treeLanes : rowsPerBlock * treeThreads;
+  }
   // Distance in LDS between feature f and f+1 of one row, in the units node offsets use.
   uint32_t FeatureStride() const {
     if (kernel == Kernel::kTreeParallel) return 4u;
@@ -49,7 +52,15 @@ struct PackedModel {
   uint32_t maxGroupNodes = 0;
 
   uint32_t PadFeatureOffset() const;
-  uint32_t GroupRegionBytes() const { return maxGroupNodes * kNodeBytes; }
+  // LDS bytes of the tree-group region (regressors reuse it for the tree threads' cross-wave pass).
+  uint32_t GroupRegionBytes() const {
+    uint32_t bytes = maxGroupNodes * kNodeBytes;
+    if (plan.kernel == LaunchPlan::Kernel::kRowParallelLds && plan.treeThreads > 1 && numClasses == 0)
+      bytes = bytes > (uint32_t)plan.ThreadsPerBlock() * 8u ? bytes : (uint32_t)plan.ThreadsPerBlock() * 8u;
+    return (bytes + 15u) & ~15u;
+  }
+  // How many partial sums per (row, class) the walk kernel leaves for the finalize kernel.
+  int32_t PartialCount() const { return plan.treeSlices; }
   size_t RowTileBytes() const;
   size_t LdsBytes() const; // row tile + the largest group (+ reduction scratch)
 };

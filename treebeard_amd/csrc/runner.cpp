@@ -94,7 +94,7 @@ void InferenceRunner::Repack(const LaunchPlan &plan) {
 
 void InferenceRunner::EnsurePartial(int64_t rows) {
   if (!NeedsFinalize()) return;
-  const size_t need = (size_t)m_model.plan.treeSlices * (size_t)rows * (size_t)std::max(1, m_forest.numClasses) * sizeof(double);
+  const size_t need = (size_t)m_model.PartialCount() * (size_t)rows * (size_t)std::max(1, m_forest.numClasses) * sizeof(double);
   if (need <= m_partialBytes) return;
   Check(hipStreamSynchronize(m_stream), "hipStreamSynchronize");
   (void)hipFree(m_dPartial);
@@ -115,8 +115,7 @@ hipError_t InferenceRunner::LaunchWalk(const WalkParams &p) const {
   const LaunchPlan &plan = m_model.plan;
   if (plan.kernel == LaunchPlan::Kernel::kTreeParallel)
     return LaunchWalkTreeParallel(p, plan.interleave, m_model.LdsBytes(), m_stream);
-  return LaunchWalkRowsLds(p, plan.rowsPerBlock, plan.interleave, plan.featureOffsetInWords, m_model.LdsBytes(),
-                           m_stream);
+  return LaunchWalkRowsLds(p, plan.interleave, plan.featureOffsetInWords, m_model.LdsBytes(), m_stream);
 }
 
 WalkParams InferenceRunner::MakeWalkParams(const float *deviceInputs, int64_t rows) const {
@@ -126,7 +125,8 @@ WalkParams InferenceRunner::MakeWalkParams(const float *deviceInputs, int64_t ro
   p.s.numClasses = m_forest.numClasses;
   p.s.numGroups = (int32_t)m_model.groups.size();
   p.s.treeSlices = m_model.plan.treeSlices;
-  p.s.groupRegionBytes = (uint32_t)m_model.maxGroupNodes * kNodeBytes;
+  p.s.groupRegionBytes = m_model.GroupRegionBytes();
+  p.s.treeThreads = m_model.plan.treeThreads;
   p.s.transform = m_forest.transform == Transform::kSigmoid ? 1 : 0;
   p.s.numTrees = (int32_t)m_forest.trees.size();
   p.s.rowsPerBlock = m_model.plan.rowsPerBlock;
@@ -158,7 +158,7 @@ void InferenceRunner::Launch(const float *deviceInputs, int64_t rows, float *out
     f.partial = m_dPartial;
     f.rows = rows;
     f.numClasses = m_forest.numClasses;
-    f.treeSlices = m_model.plan.treeSlices;
+    f.treeSlices = m_model.PartialCount();
     f.initialValue = m_forest.initialValue;
     f.transform = p.s.transform;
     f.out = out;
@@ -238,7 +238,7 @@ void InferenceRunner::TimeKernels(const float *deviceInputs, void *deviceResults
     f.partial = m_dPartial;
     f.rows = rows;
     f.numClasses = m_forest.numClasses;
-    f.treeSlices = m_model.plan.treeSlices;
+    f.treeSlices = m_model.PartialCount();
     f.initialValue = m_forest.initialValue;
     f.transform = p.s.transform;
     if (m_forest.numClasses > 0) f.classOut = static_cast<int8_t *>(deviceResults);
@@ -266,8 +266,13 @@ double InferenceRunner::AutoTune(const float *deviceInputs, int64_t rows) {
         continue; // plan cannot hold this model
       }
       double w = 0, f = 0;
-      TimeKernels(deviceInputs, out, rows, 1, &w, &f); // warm-up
-      TimeKernels(deviceInputs, out, rows, 3, &w, &f);
+      try {
+        TimeKernels(deviceInputs, out, rows, 1, &w, &f); // warm-up
+        TimeKernels(deviceInputs, out, rows, 3, &w, &f);
+      } catch (const Error &) {
+        (void)hipGetLastError(); // plan the launcher rejects (e.g. too few lanes to prefetch a group)
+        continue;
+      }
       if (w + f < bestMs) {
         bestMs = w + f;
         best = m_model.plan;
@@ -286,7 +291,8 @@ std::string InferenceRunner::DescribePlan() const {
   std::ostringstream os;
   const LaunchPlan &p = m_model.plan;
   os << "kernel=" << (p.kernel == LaunchPlan::Kernel::kTreeParallel ? "tree_parallel" : "rows_lds")
-     << " rowsPerBlock=" << p.rowsPerBlock << " treeLanes=" << p.treeLanes << " interleave=" << p.interleave
+     << " rowsPerBlock=" << p.rowsPerBlock << " treeThreads=" << p.treeThreads << " treeLanes=" << p.treeLanes
+     << " interleave=" << p.interleave
      << " groupBytes=" << p.groupBytes << " treeSlices=" << p.treeSlices
      << " offsetsInWords=" << (p.featureOffsetInWords ? 1 : 0) << " groups=" << m_model.groups.size()
      << " bundles=" << m_model.bundles.size() << " nodes=" << m_model.nodes.size()

@@ -330,7 +330,8 @@ int32_t tbmi_autotune(intptr_t h, const float *in, int64_t rows, double *bestMs)
   return Guard([&] { double ms = Runner(h)->AutoTune(in, rows); if (bestMs) *bestMs = ms; return 0; }, -1);
 }
 
-int32_t tbmi_set_plan(intptr_t h, int32_t rowsPerBlock, int32_t interleave, int32_t groupBytes, int32_t treeSlices) {
+int32_t tbmi_set_plan(intptr_t h, int32_t rowsPerBlock, int32_t treeThreads, int32_t interleave, int32_t groupBytes,
+                      int32_t treeSlices) {
   return Guard(
       [&] {
         InferenceRunner *r = Runner(h);
@@ -338,6 +339,7 @@ int32_t tbmi_set_plan(intptr_t h, int32_t rowsPerBlock, int32_t interleave, int3
         plan.kernel = LaunchPlan::Kernel::kRowParallelLds;
         plan.treeLanes = 1;
         if (rowsPerBlock > 0) plan.rowsPerBlock = rowsPerBlock;
+        plan.treeThreads = treeThreads > 0 ? treeThreads : 1;
         if (interleave > 0) plan.interleave = interleave;
         if (groupBytes > 0) plan.groupBytes = groupBytes;
         if (treeSlices > 0) plan.treeSlices = treeSlices;
@@ -357,10 +359,12 @@ int32_t tbmi_set_tree_parallel_plan(intptr_t h, int32_t rowsPerBlock, int32_t tr
         LaunchPlan plan = r->Model().plan;
         plan.kernel = LaunchPlan::Kernel::kTreeParallel;
         plan.featureOffsetInWords = false;
+        plan.treeThreads = 1;
         plan.rowsPerBlock = rowsPerBlock;
         plan.treeLanes = treeLanes;
         plan.interleave = interleave > 0 ? interleave : 1;
         if (groupBytes > 0) plan.groupBytes = groupBytes;
+        else plan.groupBytes = std::min(plan.groupBytes, 256 * plan.ThreadsPerBlock());
         if (treeSlices > 0) plan.treeSlices = treeSlices;
         r->Repack(plan);
         return 0;

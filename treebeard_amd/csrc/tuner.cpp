@@ -22,21 +22,6 @@ bool RowTileFits(int32_t numFeatures, int32_t rowsPerBlock, int32_t ldsBytes, bo
   return true;
 }
 
-void FitGroupBytes(LaunchPlan &plan, const Forest &forest, const DeviceLimits &limits, int blocksPerCu) {
-  const int64_t rowTile = (int64_t)(forest.numFeatures + 1) * plan.rowsPerBlock * 4;
-  int64_t perBlock = limits.ldsBytesPerBlock / blocksPerCu;
-  int64_t group = std::min<int64_t>(65536, perBlock - rowTile);
-  // the biggest tree has to fit a group (+ null leaf + alignment pad)
-  int64_t biggest = 0;
-  for (auto &t : forest.trees) biggest = std::max<int64_t>(biggest, (int64_t)t.NumNodes());
-  const int64_t need = (biggest + 2) * kNodeBytes;
-  if (group < need) group = std::min<int64_t>(65536, std::min<int64_t>(limits.ldsBytesPerBlock - rowTile, std::max<int64_t>(need, 16384)));
-  plan.groupBytes = (int32_t)(group & ~15);
-}
-
-} // namespace
-
-namespace {
 
 int64_t BiggestTreeNodes(const Forest &forest) {
   int64_t biggest = 0;
@@ -69,6 +54,8 @@ LaunchPlan ChooseTreeParallelPlan(const Forest &forest, int64_t batchSize, const
   // narrow rows leave LDS for bigger groups
   const int64_t rowTile = rowBytes * plan.rowsPerBlock;
   group = std::max<int64_t>(group, std::min<int64_t>(65536, (limits.ldsBytesPerBlock / 2 - rowTile - reserve)));
+  group = std::min<int64_t>(group, 256LL * plan.ThreadsPerBlock()); // 16 prefetch registers of 16 bytes per lane
+  if (group < need) throw Error("the biggest tree does not fit the group prefetch registers of this block shape");
   plan.groupBytes = (int32_t)(std::min<int64_t>(group, 65536) & ~15);
 
   const int64_t rowBlocks = std::max<int64_t>(1, (batchSize + plan.rowsPerBlock - 1) / plan.rowsPerBlock);
@@ -102,37 +89,52 @@ LaunchPlan ChoosePlan(const Forest &forest, int64_t batchSize, const GPUAutoSche
   LaunchPlan plan;
   plan.kernel = LaunchPlan::Kernel::kRowParallelLds;
 
+  // Shape that measured best on MI355X: blocks of 1024 lanes (16 waves), two blocks per CU
+  // (full occupancy), each block 256 rows x 4 tree threads when the row tile allows it, and the
+  // tree group as large as half the LDS leaves room for.
+  const int32_t halfLds = limits.ldsBytesPerBlock / 2;
   int32_t rb = 256;
   if (ov && ov->numRowsPerTB > 0) rb = std::max(64, FloorPow2(ov->numRowsPerTB));
-  if (batchSize > 0 && batchSize < rb) rb = std::max<int32_t>(64, FloorPow2(std::max<int64_t>(batchSize, 1) * 2 - 1));
   bool words = false;
-  while (rb > 64 && !RowTileFits(forest.numFeatures, rb, limits.ldsBytesPerBlock, &words)) rb /= 2;
-  if (!RowTileFits(forest.numFeatures, rb, limits.ldsBytesPerBlock, &words))
-    throw Error("row tile of " + std::to_string(forest.numFeatures) + " features does not fit LDS");
+  auto fits = [&](int32_t r) { return RowTileFits(forest.numFeatures, r, halfLds + 8192, &words); };
+  while (rb > 64 && !fits(rb)) rb /= 2;
+  int32_t budget = halfLds;
+  if (!fits(rb)) { // one block per CU
+    budget = limits.ldsBytesPerBlock;
+    if (!RowTileFits(forest.numFeatures, rb, budget, &words))
+      throw Error("row tile of " + std::to_string(forest.numFeatures) + " features does not fit LDS");
+  }
   plan.rowsPerBlock = rb;
   plan.featureOffsetInWords = words;
+  plan.treeThreads = std::max(1, std::min(8, 1024 / rb));
+  if (ov && ov->numTreeThreads > 0) plan.treeThreads = std::max(1, std::min(ov->numTreeThreads, 1024 / rb));
 
   plan.interleave = 4;
   if (ov && ov->treeWalkInterleaveFactor > 0)
     plan.interleave = std::min(kMaxInterleave, FloorPow2(ov->treeWalkInterleaveFactor));
 
-  FitGroupBytes(plan, forest, limits, /*blocksPerCu=*/2);
+  const int64_t rowTile = (int64_t)(forest.numFeatures + 1) * rb * 4;
+  const int64_t need = (BiggestTreeNodes(forest) + 2) * kNodeBytes;
+  if (need > 65536) throw Error("a tree does not fit one LDS tree group");
+  const int64_t meet = forest.numClasses > 0 ? (int64_t)rb * plan.treeThreads * 8 : 0; // cross-wave pass
+  // (LDS is handed out in coarse pieces: leave slack or the second block will not fit)
+  int64_t group = std::min<int64_t>(65536, budget - rowTile - meet - 2048);
+  if (group < need) group = std::min<int64_t>(65536, limits.ldsBytesPerBlock - rowTile - meet - 2048);
+  group = std::min<int64_t>(group, 256LL * rb * plan.treeThreads); // 16 prefetch registers of 16 bytes per lane
+  if (group < need) throw Error("the biggest tree does not fit LDS next to the row tile");
+  plan.groupBytes = (int32_t)(group & ~15);
 
   // Tree slices: when the batch alone cannot fill the chip, blocks share a row
   // tile and split the tree groups between them.
   const int64_t rowBlocks = std::max<int64_t>(1, (batchSize + rb - 1) / rb);
-  int64_t totalNodes = (int64_t)forest.NumNodes();
-  int64_t groups = std::max<int64_t>(1, (totalNodes * kNodeBytes + plan.groupBytes - 1) / plan.groupBytes);
+  const int64_t totalBytes = (int64_t)forest.NumNodes() * kNodeBytes;
+  int64_t groups = std::max<int64_t>(1, (totalBytes + plan.groupBytes - 1) / plan.groupBytes);
   int64_t slices = 1;
   const int64_t wantBlocks = 2LL * limits.computeUnits;
-  if (rowBlocks < wantBlocks) slices = std::min<int64_t>(groups, (wantBlocks + rowBlocks - 1) / rowBlocks);
-  if (ov && ov->numTreeThreads > 0) slices = std::min<int64_t>(groups, ov->numTreeThreads);
-  if (slices > 1) {
-    // more, smaller groups so that every slice has at least one
-    int64_t perSlice = (totalNodes * kNodeBytes + slices - 1) / slices + 4096;
-    int64_t biggest = 0;
-    for (auto &t : forest.trees) biggest = std::max<int64_t>(biggest, (int64_t)t.NumNodes());
-    perSlice = std::max<int64_t>(perSlice, (biggest + 2) * kNodeBytes);
+  if (rowBlocks < wantBlocks) slices = (wantBlocks + rowBlocks - 1) / rowBlocks;
+  slices = std::min<int64_t>(slices, std::max<int64_t>(1, totalBytes / 16384)); // >= 16 KB of trees per slice
+  if (slices > groups) { // more, smaller groups so that every slice has one
+    int64_t perSlice = std::max<int64_t>((totalBytes + slices - 1) / slices + 4096, need);
     if (perSlice < plan.groupBytes) plan.groupBytes = (int32_t)((perSlice + 15) & ~15);
   }
   plan.treeSlices = (int32_t)std::max<int64_t>(1, slices);
@@ -155,28 +157,32 @@ std::vector<LaunchPlan> CandidatePlans(const Forest &forest, int64_t batchSize, 
       }
     return out;
   }
+  const int64_t need = (BiggestTreeNodes(forest) + 2) * kNodeBytes;
   for (int32_t rb : {64, 128, 256, 512})
-    for (int32_t k : {2, 4, 8})
-      for (int blocksPerCu : {1, 2, 3}) {
-        bool words = false;
-        if (!RowTileFits(forest.numFeatures, rb, limits.ldsBytesPerBlock / blocksPerCu, &words)) continue;
-        LaunchPlan p = base;
-        p.rowsPerBlock = rb;
-        p.featureOffsetInWords = words;
-        p.interleave = k;
-        FitGroupBytes(p, forest, limits, blocksPerCu);
-        if ((int64_t)(forest.numFeatures + 1) * rb * 4 + p.groupBytes > limits.ldsBytesPerBlock) continue;
-        const int64_t rowBlocks = std::max<int64_t>(1, (batchSize + rb - 1) / rb);
-        if (base.treeSlices > 1) {
-          int64_t groups = std::max<int64_t>(1, ((int64_t)forest.NumNodes() * kNodeBytes + p.groupBytes - 1) / p.groupBytes);
-          p.treeSlices = (int32_t)std::min<int64_t>(groups, std::max<int64_t>(1, 2LL * limits.computeUnits / rowBlocks));
+    for (int32_t tt : {1, 2, 4, 8})
+      for (int32_t k : {2, 4, 8})
+        for (int blocksPerCu : {1, 2, 3}) {
+          if (rb * tt > 1024) continue;
+          bool words = false;
+          const int32_t budget = limits.ldsBytesPerBlock / blocksPerCu;
+          if (!RowTileFits(forest.numFeatures, rb, budget + 8192, &words)) continue;
+          LaunchPlan p = base;
+          p.rowsPerBlock = rb;
+          p.treeThreads = tt;
+          p.featureOffsetInWords = words;
+          p.interleave = k;
+          const int64_t rowTile = (int64_t)(forest.numFeatures + 1) * rb * 4;
+          int64_t group = std::min<int64_t>(65536, budget - rowTile - (forest.numClasses > 0 ? (int64_t)rb * tt * 8 : 0) - 2048);
+          group = std::min<int64_t>(group, 256LL * rb * tt); // 16 prefetch registers of 16 bytes per lane
+          if (group < need || group < 8192) continue;
+          if (base.treeSlices > 1) group = std::min<int64_t>(group, base.groupBytes);
+          p.groupBytes = (int32_t)(group & ~15);
+          bool dup = false;
+          for (auto &q : out)
+            dup = dup || (q.rowsPerBlock == p.rowsPerBlock && q.treeThreads == p.treeThreads &&
+                          q.interleave == p.interleave && q.groupBytes == p.groupBytes);
+          if (!dup) out.push_back(p);
         }
-        bool dup = false;
-        for (auto &q : out)
-          dup = dup || (q.rowsPerBlock == p.rowsPerBlock && q.interleave == p.interleave &&
-                        q.groupBytes == p.groupBytes && q.treeSlices == p.treeSlices);
-        if (!dup) out.push_back(p);
-      }
   return out;
 }
 

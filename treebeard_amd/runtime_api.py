@@ -58,7 +58,7 @@ SIGNATURES = {
     "tbmi_time_kernels": (c_i32, [c_ip, c_vp, c_vp, c_i64, c_i32, ctypes.POINTER(ctypes.c_double),
                                   ctypes.POINTER(ctypes.c_double)]),
     "tbmi_autotune": (c_i32, [c_ip, c_vp, c_i64, ctypes.POINTER(ctypes.c_double)]),
-    "tbmi_set_plan": (c_i32, [c_ip, c_i32, c_i32, c_i32, c_i32]),
+    "tbmi_set_plan": (c_i32, [c_ip, c_i32, c_i32, c_i32, c_i32, c_i32]),
     "tbmi_set_tree_parallel_plan": (c_i32, [c_ip, c_i32, c_i32, c_i32, c_i32, c_i32]),
     "tbmi_describe_plan": (c_i32, [c_ip, c_cp, c_i32]),
     "tbmi_num_trees": (c_i32, [c_ip]),

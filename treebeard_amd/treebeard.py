@@ -296,9 +296,9 @@ class TreebeardInferenceRunner:
                  "tbmi_autotune")
         return best.value
 
-    def set_plan(self, rows_per_block=0, interleave=0, group_bytes=0, tree_slices=0):
-        self._rc(_lib().tbmi_set_plan(self.inferenceRunner, rows_per_block, interleave, group_bytes, tree_slices),
-                 "tbmi_set_plan")
+    def set_plan(self, rows_per_block=0, tree_threads=1, interleave=0, group_bytes=0, tree_slices=0):
+        self._rc(_lib().tbmi_set_plan(self.inferenceRunner, rows_per_block, tree_threads, interleave, group_bytes,
+                                      tree_slices), "tbmi_set_plan")
 
     def set_tree_parallel_plan(self, rows_per_block, tree_lanes, interleave=1, group_bytes=0, tree_slices=0):
         self._rc(_lib().tbmi_set_tree_parallel_plan(self.inferenceRunner, rows_per_block, tree_lanes, interleave,
