@@ -33,6 +33,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--autotune", action="store_true", help="timed launch-plan search before measuring")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU-baseline duration")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
+                    help="also run one plain device copy of this many MiB (counter calibration for rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this engine runs on ONE GPU (rows shard trivially; see DESIGN.md) - use --gpus 1")
@@ -53,6 +55,12 @@ def main():
     out = torch.zeros(rows, dtype=torch.int8 if multiclass else torch.float32, device="cuda")
     if args.autotune:
         runner.autotune(dx.data_ptr(), rows)
+    if args.copy_calibration:
+        # a plain device copy of known size: scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run
+        a = torch.empty(args.copy_calibration << 20, dtype=torch.uint8, device="cuda")
+        b = torch.empty_like(a)
+        b.copy_(a)
+        torch.cuda.synchronize()
 
     for _ in range(args.warmup):
         runner.run_device(dx.data_ptr(), out.data_ptr(), rows)
