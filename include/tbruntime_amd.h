@@ -121,9 +121,11 @@ TBAMD_EXPORT int32_t tbmi_run_device_multiclass(intptr_t runner, const float *de
  * int32 [rows][numTrees] in device memory. */
 TBAMD_EXPORT int32_t tbmi_dump_leaf_ids(intptr_t runner, const float *deviceInputs, int32_t *deviceLeafIds,
                                         int64_t rows);
-/* Average kernel durations (ms) over `runs` launches, measured with HIP events on the runner's stream. */
+/* Average kernel durations (ms) over `runs` launches each, measured with HIP events on the runner's stream:
+ * the walk kernel, the finalize kernel and the rank-quantisation kernel (0 when the plan has none). */
 TBAMD_EXPORT int32_t tbmi_time_kernels(intptr_t runner, const float *deviceInputs, void *deviceResults,
-                                       int64_t rows, int32_t runs, double *walkMs, double *finalizeMs);
+                                       int64_t rows, int32_t runs, double *walkMs, double *finalizeMs,
+                                       double *binMs);
 /* Timed search over launch plans on the given rows; keeps the fastest plan. */
 TBAMD_EXPORT int32_t tbmi_autotune(intptr_t runner, const float *deviceInputs, int64_t rows, double *bestMs);
 /* Pins the row-parallel kernel: rowsPerBlock rows per block, treeThreads lanes per row (in different
@@ -134,6 +136,9 @@ TBAMD_EXPORT int32_t tbmi_set_plan(intptr_t runner, int32_t rowsPerBlock, int32_
 /* Pins the tree-parallel kernel: rowsPerBlock rows per block, treeLanes lanes per row. */
 TBAMD_EXPORT int32_t tbmi_set_tree_parallel_plan(intptr_t runner, int32_t rowsPerBlock, int32_t treeLanes,
                                                  int32_t interleave, int32_t groupBytes, int32_t treeSlices);
+/* Pins the row-parallel kernel on rank-quantised rows (64 rows per block, one byte per feature value). */
+TBAMD_EXPORT int32_t tbmi_set_quantized_plan(intptr_t runner, int32_t treeThreads, int32_t interleave,
+                                             int32_t groupBytes, int32_t treeSlices);
 TBAMD_EXPORT int32_t tbmi_describe_plan(intptr_t runner, char *buffer, int32_t length);
 TBAMD_EXPORT int32_t tbmi_num_trees(intptr_t runner);
 TBAMD_EXPORT int32_t tbmi_num_classes(intptr_t runner);

@@ -231,6 +231,47 @@ def test_small_batches_pick_the_tree_parallel_kernel(synth_model, k, rows):
     check_against_oracle(runner, forest, x)
 
 
+def coarse_model(path, num_features, num_trees, num_class, seed):
+    """Trees whose thresholds come from a grid of 40 values per feature (so ranks fit one byte)."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    grid = np.round(rng.normal(size=(40, num_features)), 2).astype(np.float32)
+    trees = [synth._grow_tree(rng, 7, lambda d, s: 0.85, lambda: (lambda f: (f, grid[rng.integers(0, 40), f]))(rng.integers(0, num_features)),
+                              lambda: rng.normal(0, 0.1)) for _ in range(num_trees)]
+    synth.write_xgboost_json(path, trees, num_features, objective="multi:softmax" if num_class else "reg:squarederror",
+                             num_class=num_class, tree_info=[t % num_class for t in range(num_trees)] if num_class else None)
+    return grid
+
+
+@pytest.mark.parametrize("plan", [(8, 4, 0, 1), (16, 1, 16384, 1), (4, 2, 32768, 3), (1, 8, 16384, 1)])
+@pytest.mark.parametrize("model", ["config4", "coarse_regression", "coarse_multiclass"])
+def test_rank_quantised_plans_agree(synth_model, tmp_path, model, plan):
+    """Rows replaced by one-byte ranks among each feature's thresholds: leaf selection must not change."""
+    if model == "config4":
+        path, rows = synth_model(4), 333
+        x = synth.CONFIGS[4].batch_rows(rows, seed_offset=5)
+    else:
+        path, rows = str(tmp_path / "coarse.json"), 1500
+        grid = coarse_model(path, 37, 120, 5 if model == "coarse_multiclass" else 0, seed=17)
+        rng = np.random.default_rng(3)
+        x = np.round(rng.normal(size=(rows, 37)), 2).astype(np.float32)     # many values equal to thresholds
+    forest = model_io.load_xgboost_json(path)
+    thr, feat, left, _ = forest.tree(0)
+    for i in np.nonzero(left != -1)[0][:20]:
+        x[int(i) % rows, feat[i]] = np.float32(thr[i])
+    x[3, :] = np.inf
+    x[4, :] = -np.inf
+    runner = make_runner(path, rows)
+    runner.set_quantized_plan(*plan)
+    assert "quantizedRows=1" in runner.describe_plan()
+    check_against_oracle(runner, forest, x)
+
+
+def test_rank_quantisation_is_refused_when_a_feature_has_too_many_thresholds(synth_model):
+    runner = make_runner(synth_model(2), 512)
+    with pytest.raises(RuntimeError, match="254 distinct thresholds"):
+        runner.set_quantized_plan(8, 4, 0, 1)
+
+
 def test_gpu_auto_schedule_options_are_honoured(synth_model):
     gpu = treebeard.GPUAutoScheduleOptions.Construct(num_rows_per_TB=64, num_tree_threads=10,
                                                      tree_walk_interleave_factor=2, cache_rows=True)

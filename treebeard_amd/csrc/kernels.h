@@ -51,9 +51,13 @@ struct FinalizeParams {
 };
 
 // Row-parallel walk over LDS-staged tree groups: block = s.rowsPerBlock * s.treeThreads lanes.
-// `interleave` in {1,2,4,8}; `featureOffsetInWords` selects how node feature offsets are scaled.
-hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, bool featureOffsetInWords, size_t ldsBytes,
-                             hipStream_t stream);
+// `interleave` in {1,2,4,8}; `tileMode`: 0 f32 tile with byte offsets, 1 f32 tile with offsets in units of
+// 4 bytes, 2 one-byte rank tile (p.x then points at the output of LaunchBinRows; 64 rows per block).
+hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, int tileMode, size_t ldsBytes, hipStream_t stream);
+// Rank-quantises rows x[rows][numFeatures] into ranks[ceil(rows/64)][numFeatures][64] (bytes) with the
+// packer's threshold table ([chunk][k][chunkFeatures], NaN padded, tableDepth = 2^n - 1).
+hipError_t LaunchBinRows(const float *x, const float *table, uint8_t *ranks, int64_t rows, int numFeatures,
+                         int tableDepth, int chunkFeatures, hipStream_t stream);
 // Tree-parallel walk: s.rowsPerBlock rows per block (row-major in LDS),
 // s.treeLanes lanes per row; block = rowsPerBlock * treeLanes lanes.
 hipError_t LaunchWalkTreeParallel(const WalkParams &p, int interleave, size_t ldsBytes, hipStream_t stream);

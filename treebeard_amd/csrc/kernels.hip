@@ -25,6 +25,15 @@ typedef const __attribute__((address_space(3))) U32x2 *LdsNodePtr;
 typedef const __attribute__((address_space(3))) float *LdsFloatPtr;
 __device__ __forceinline__ U32x2 LdsLoadNode(uint32_t address) { return *(LdsNodePtr)(uintptr_t)address; }
 __device__ __forceinline__ float LdsLoadFloat(uint32_t address) { return *(LdsFloatPtr)(uintptr_t)address; }
+typedef const __attribute__((address_space(3))) uint8_t *LdsBytePtr;
+__device__ __forceinline__ uint32_t LdsLoadByte(uint32_t address) { return *(LdsBytePtr)(uintptr_t)address; }
+
+// How a node's 16-bit feature offset addresses the row tile of the row-parallel kernel.
+enum RowTileMode : int {
+  kTileF32Bytes = 0, // f32 tile, offset in bytes
+  kTileF32Words = 1, // f32 tile, offset in units of 4 bytes (tiles above 64 KB)
+  kTileRankU8 = 2    // one-byte rank tile (rank-quantised rows), offset in units of 4 bytes
+};
 
 
 // Copies the block's rows (contiguous, row-major in global memory) into the LDS tile.
@@ -105,7 +114,7 @@ __device__ __forceinline__ void StageRows(const float *__restrict__ src, int val
 // without growing the row tile; their sums meet in an LDS cross-wave pass.
 // Sums are kept in double; trees are added in packed order.
 // ---------------------------------------------------------------------------
-template <int K, int PF, bool kOffsetsInWords, bool kDump>
+template <int K, int PF, int kMode, bool kDump>
 __global__ void __launch_bounds__(1024)
 WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16,
                   const DeviceBundle *__restrict__ bundles, const DeviceGroup *__restrict__ groups,
@@ -127,12 +136,35 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
   const int64_t remaining = s.rows - row0;
   const int valid = remaining < RB ? (int)remaining : RB;
 
-  float *rowTile = reinterpret_cast<float *>(lds + s.groupRegionBytes);
-
-  // Stage the block's rows: coalesced reads of the contiguous row-major tile, transposed writes.
-  StageRows<true>(x + row0 * F, valid, RB, F, 0, rowTile, tid, threads);
-  for (int i = tid; i < RB; i += threads) rowTile[F * RB + i] = -INFINITY; // pad feature: keeps leaves in place
-  const uint32_t column = s.groupRegionBytes + (uint32_t)lane * 4u; // LDS address of this row's feature 0
+  uint32_t column; // LDS address of this row's feature 0
+  if (kMode == kTileRankU8) {
+    // Rank-quantised rows arrive already tiled ([row block][feature][row], one byte each): plain copy.
+    typedef uint32_t Piece __attribute__((ext_vector_type(4)));
+    const Piece *src = reinterpret_cast<const Piece *>(reinterpret_cast<const uint8_t *>(x) + (int64_t)blockIdx.x * F * RB);
+    Piece *dst = reinterpret_cast<Piece *>(lds + s.groupRegionBytes);
+    const int pieces = (F * RB) >> 4;
+    for (int base = 0; base < pieces; base += threads * kStageUnroll) {
+      Piece v[kStageUnroll];
+#pragma unroll
+      for (int u = 0; u < kStageUnroll; ++u) {
+        const int idx = base + u * threads + tid;
+        v[u] = src[idx < pieces ? idx : pieces - 1];
+      }
+#pragma unroll
+      for (int u = 0; u < kStageUnroll; ++u) {
+        const int idx = base + u * threads + tid;
+        if (idx < pieces) dst[idx] = v[u];
+      }
+    }
+    for (int i = tid; i < RB; i += threads) lds[s.groupRegionBytes + (uint32_t)F * RB + i] = 0; // pad feature: rank 0
+    column = s.groupRegionBytes + (uint32_t)lane;
+  } else {
+    float *rowTile = reinterpret_cast<float *>(lds + s.groupRegionBytes);
+    // Stage the block's rows: coalesced reads of the contiguous row-major tile, transposed writes.
+    StageRows<true>(x + row0 * F, valid, RB, F, 0, rowTile, tid, threads);
+    for (int i = tid; i < RB; i += threads) rowTile[F * RB + i] = -INFINITY; // pad feature: keeps leaves in place
+    column = s.groupRegionBytes + (uint32_t)lane * 4u;
+  }
 
   const int slice = blockIdx.y;
   const int gBegin = (int)(((int64_t)s.numGroups * slice) / s.treeSlices);
@@ -143,7 +175,8 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
   // LDS cross-wave pass: the tree threads of a row leave their sums here and tree thread 0 adds
   // them in thread order.  Classifiers meet at class boundaries, while a tree group is live, so
   // their meeting area sits behind the row tile; otherwise the (then idle) group region is used.
-  double *meet = reinterpret_cast<double *>(C > 0 ? lds + s.groupRegionBytes + (uint32_t)(F + 1) * RB * 4u : lds);
+  double *meet = reinterpret_cast<double *>(
+      C > 0 ? lds + ((s.groupRegionBytes + (uint32_t)(F + 1) * RB * (kMode == kTileRankU8 ? 1u : 4u) + 7u) & ~7u) : lds);
 
   double acc = 0.0;
   int curClass = 0;
@@ -220,9 +253,11 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
 #pragma unroll
           for (int k = 0; k < K; ++k) {
             const U32x2 node = LdsLoadNode(addr[k]);
-            const uint32_t off = kOffsetsInWords ? (node.y & 0xFFFFu) << 2 : (node.y & 0xFFFFu);
-            const float xv = LdsLoadFloat(column + off);
-            addr[k] = (node.y >> 16) + (xv < AsFloat(node.x) ? 0u : kNodeBytes);
+            const uint32_t off = kMode == kTileF32Bytes ? (node.y & 0xFFFFu) : (node.y & 0xFFFFu) << 2;
+            bool left;
+            if (kMode == kTileRankU8) left = LdsLoadByte(column + off) <= node.x; // rank <= threshold index
+            else left = LdsLoadFloat(column + off) < AsFloat(node.x);
+            addr[k] = (node.y >> 16) + (left ? 0u : kNodeBytes);
           }
         }
 #pragma unroll
@@ -413,6 +448,77 @@ WalkTreeParallelKernel(const float *__restrict__ x, const uint4 *__restrict__ no
 }
 
 // ---------------------------------------------------------------------------
+// Rank quantisation of the rows.  For every (row, feature) the kernel counts how many of the
+// feature's sorted distinct split thresholds are <= the value (NaN counts as 255, which no node
+// accepts as "left") and writes the count as one byte into the tile layout the row-parallel kernel
+// copies verbatim: [block of 64 rows][feature][row].  The block owns a chunk of features, whose
+// threshold table sits in LDS as [k][feature], and walks the row blocks.  Four consecutive lanes
+// share a feature and take 16 rows of the row block each, so a lane produces exactly one 16-byte
+// piece of the tile and a wave's store covers 1 KB of contiguous tile (16 features x 64 rows).
+// ---------------------------------------------------------------------------
+constexpr int kBinRows = 64;       // rows per tile = rows per block of the quantised walk
+constexpr int kBinRowsPerLane = 16;
+
+__global__ void __launch_bounds__(1024)
+BinRowsKernel(const float *__restrict__ x, const float *__restrict__ table, uint8_t *__restrict__ ranks,
+              int64_t rows, int F, int depth, int rowBlocksPerBlock) {
+  extern __shared__ __align__(16) unsigned char lds[];
+  float *tab = reinterpret_cast<float *>(lds);
+  const int tid = threadIdx.x;
+  const int FC = blockDim.x >> 2; // features per block
+  const int fl = tid >> 2;        // feature inside the chunk
+  const int sub = tid & 3;        // which 16 rows of the row block
+  const int f = blockIdx.x * FC + fl;
+  {
+    const float *src = table + (int64_t)blockIdx.x * depth * FC;
+    for (int i = tid; i < depth * FC; i += blockDim.x) tab[i] = src[i];
+  }
+  __syncthreads();
+  const int64_t numRowBlocks = (rows + kBinRows - 1) / kBinRows;
+  const int64_t rbBegin = (int64_t)blockIdx.y * rowBlocksPerBlock;
+  const int64_t rbEnd = rbBegin + rowBlocksPerBlock < numRowBlocks ? rbBegin + rowBlocksPerBlock : numRowBlocks;
+  const int fClamped = f < F ? f : F - 1;
+  const uint32_t strideBytes = (uint32_t)FC * 4u;                  // one table level
+  const uint32_t laneBytes = (uint32_t)fl * 4u;
+  const uint32_t halfBytes = (uint32_t)((depth + 1) >> 1) * strideBytes; // depth = 2^n - 1
+  int shift = 0;
+  while ((1u << shift) < strideBytes) ++shift;                     // FC is a power of two
+  for (int64_t rb = rbBegin; rb < rbEnd; ++rb) {
+    const int64_t rowBase = rb * kBinRows + sub * kBinRowsPerLane;
+    float v[kBinRowsPerLane];
+#pragma unroll
+    for (int u = 0; u < kBinRowsPerLane; ++u) { // all loads in flight; rows past the batch re-read the last row
+      const int64_t row = rowBase + u;
+      v[u] = x[(row < rows ? row : rows - 1) * F + fClamped];
+    }
+    // branch-free binary search on byte offsets, the 16 rows side by side so that their LDS reads overlap
+    uint32_t pos[kBinRowsPerLane];
+#pragma unroll
+    for (int u = 0; u < kBinRowsPerLane; ++u) pos[u] = 0;
+    for (uint32_t step = halfBytes; step >= strideBytes; step >>= 1) {
+      const uint32_t probe = step - strideBytes + laneBytes;
+#pragma unroll
+      for (int u = 0; u < kBinRowsPerLane; ++u) pos[u] += LdsLoadFloat(pos[u] + probe) <= v[u] ? step : 0u;
+    }
+    uint32_t packed[kBinRowsPerLane / 4];
+#pragma unroll
+    for (int i = 0; i < kBinRowsPerLane / 4; ++i) packed[i] = 0;
+#pragma unroll
+    for (int u = 0; u < kBinRowsPerLane; ++u) {
+      uint32_t rank = pos[u] >> shift;
+      if (v[u] != v[u]) rank = 255u;
+      if (rowBase + u >= rows) rank = 0u;
+      packed[u >> 2] |= rank << (8 * (u & 3));
+    }
+    if (f < F) {
+      typedef uint32_t Piece __attribute__((ext_vector_type(4)));
+      *reinterpret_cast<Piece *>(ranks + (rb * F + f) * kBinRows + sub * kBinRowsPerLane) =
+          Piece{packed[0], packed[1], packed[2], packed[3]};
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Sums the tree-slice partials of each row (in slice order, starting from the
 // initial value), then applies the output transform.  Multiclass rows get the
 // arg-max of the f32 per-class sums with the generated-code tie rule (running
@@ -458,7 +564,7 @@ __global__ void __launch_bounds__(256) FinalizeKernel(const FinalizeParams p) {
   }
 }
 
-template <int K, int PF, bool W>
+template <int K, int PF, int W>
 hipError_t LaunchWalkKP(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
   if (p.leafIds) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&WalkRowsLdsKernel<K, PF, W, true>),
@@ -476,7 +582,7 @@ hipError_t LaunchWalkKP(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBy
   return hipGetLastError();
 }
 
-template <int K, bool W>
+template <int K, int W>
 hipError_t LaunchWalkK(const WalkParams &p, int prefetch, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
   if (prefetch <= 4) return LaunchWalkKP<K, 4, W>(p, grid, block, ldsBytes, stream);
   if (prefetch <= 8) return LaunchWalkKP<K, 8, W>(p, grid, block, ldsBytes, stream);
@@ -484,7 +590,7 @@ hipError_t LaunchWalkK(const WalkParams &p, int prefetch, dim3 grid, dim3 block,
   return hipErrorInvalidValue;
 }
 
-template <bool W>
+template <int W>
 hipError_t LaunchWalkW(const WalkParams &p, int interleave, int prefetch, dim3 grid, dim3 block, size_t ldsBytes,
                        hipStream_t stream) {
   switch (interleave) {
@@ -498,8 +604,7 @@ hipError_t LaunchWalkW(const WalkParams &p, int interleave, int prefetch, dim3 g
 
 } // namespace
 
-hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, bool featureOffsetInWords, size_t ldsBytes,
-                             hipStream_t stream) {
+hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, int tileMode, size_t ldsBytes, hipStream_t stream) {
   if (p.s.rows <= 0) return hipSuccess;
   const int RB = p.s.rowsPerBlock, TT = p.s.treeThreads;
   if (ldsBytes > 160 * 1024 || RB < 64 || (RB & (RB - 1)) || TT < 1 || RB * TT > 1024) return hipErrorInvalidValue;
@@ -508,8 +613,14 @@ hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, bool featureOf
   // registers that hold the next tree group while the current one is walked
   const int prefetch = (int)((p.s.groupRegionBytes / 16 + RB * TT - 1) / (RB * TT));
   dim3 grid((unsigned)blocks, (unsigned)p.s.treeSlices), block((unsigned)(RB * TT));
-  return featureOffsetInWords ? LaunchWalkW<true>(p, interleave, prefetch, grid, block, ldsBytes, stream)
-                              : LaunchWalkW<false>(p, interleave, prefetch, grid, block, ldsBytes, stream);
+  switch (tileMode) {
+  case kTileF32Bytes: return LaunchWalkW<kTileF32Bytes>(p, interleave, prefetch, grid, block, ldsBytes, stream);
+  case kTileF32Words: return LaunchWalkW<kTileF32Words>(p, interleave, prefetch, grid, block, ldsBytes, stream);
+  case kTileRankU8:
+    if (RB != 64) return hipErrorInvalidValue;
+    return LaunchWalkW<kTileRankU8>(p, interleave, prefetch, grid, block, ldsBytes, stream);
+  default: return hipErrorInvalidValue;
+  }
 }
 
 namespace {
@@ -557,6 +668,28 @@ hipError_t LaunchWalkTreeParallel(const WalkParams &p, int interleave, size_t ld
   case 8: return LaunchTreeParallelK<8>(p, prefetch, grid, block, ldsBytes, stream);
   default: return hipErrorInvalidValue;
   }
+}
+
+hipError_t LaunchBinRows(const float *x, const float *table, uint8_t *ranks, int64_t rows, int numFeatures,
+                         int tableDepth, int chunkFeatures, hipStream_t stream) {
+  if (rows <= 0) return hipSuccess;
+  if (chunkFeatures != 64 && chunkFeatures != 128 && chunkFeatures != 256) return hipErrorInvalidValue;
+  const size_t ldsBytes = (size_t)tableDepth * chunkFeatures * sizeof(float);
+  if (ldsBytes > 160 * 1024) return hipErrorInvalidValue;
+  const int64_t rowBlocks = (rows + kBinRows - 1) / kBinRows;
+  const int chunks = (numFeatures + chunkFeatures - 1) / chunkFeatures;
+  // enough blocks to fill the chip, each amortising its table load over several row blocks
+  int64_t perBlock = (rowBlocks * chunks + 2047) / 2048;
+  if (perBlock < 1) perBlock = 1;
+  if (perBlock > 64) perBlock = 64;
+  const int64_t gridY = (rowBlocks + perBlock - 1) / perBlock;
+  if (gridY > 65535) return hipErrorInvalidValue;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&BinRowsKernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
+  if (e != hipSuccess) return e;
+  BinRowsKernel<<<dim3((unsigned)chunks, (unsigned)gridY), dim3((unsigned)chunkFeatures * 4u), ldsBytes, stream>>>(
+      x, table, ranks, rows, numFeatures, tableDepth, (int)perBlock);
+  return hipGetLastError();
 }
 
 hipError_t LaunchFinalize(const FinalizeParams &p, hipStream_t stream) {

@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cmath>
 #include <limits>
+#include <cstring>
 #include <numeric>
 
 namespace tbamd {
@@ -25,7 +26,9 @@ Forest NormalizeToLessThan(const Forest &forest) {
 
 uint32_t PackedModel::PadFeatureOffset() const { return (uint32_t)numFeatures * plan.FeatureStride(); }
 
-size_t PackedModel::RowTileBytes() const { return (size_t)(numFeatures + 1) * plan.rowsPerBlock * 4; }
+size_t PackedModel::RowTileBytes() const {
+  return (size_t)(numFeatures + 1) * plan.rowsPerBlock * (plan.quantizedRows ? 1 : 4);
+}
 
 size_t PackedModel::LdsBytes() const {
   size_t bytes = RowTileBytes() + (size_t)GroupRegionBytes();
@@ -35,9 +38,33 @@ size_t PackedModel::LdsBytes() const {
     bytes = (bytes + 7) & ~(size_t)7;
     bytes += waves * 8 + (size_t)plan.rowsPerBlock * (numClasses > 0 ? numClasses : 1) * 8;
   } else if (plan.treeThreads > 1 && numClasses > 0) {
+    bytes = (bytes + 7) & ~(size_t)7;
     bytes += (size_t)plan.ThreadsPerBlock() * 8; // classifiers: cross-wave pass behind the row tile
   }
   return bytes;
+}
+
+namespace {
+
+// Sorted distinct thresholds per feature of a forest already normalised to "x < t".
+std::vector<std::vector<float>> ThresholdsPerFeature(const Forest &forest) {
+  std::vector<std::vector<float>> out((size_t)forest.numFeatures);
+  for (auto &tree : forest.trees)
+    for (size_t i = 0; i < tree.NumNodes(); ++i)
+      if (!tree.IsLeaf((int32_t)i)) out[(size_t)tree.feature[i]].push_back(tree.value[i]);
+  for (auto &v : out) {
+    std::sort(v.begin(), v.end());
+    v.erase(std::unique(v.begin(), v.end()), v.end());
+  }
+  return out;
+}
+
+} // namespace
+
+int32_t MaxThresholdsPerFeature(const Forest &forest) {
+  size_t most = 0;
+  for (auto &v : ThresholdsPerFeature(NormalizeToLessThan(forest))) most = std::max(most, v.size());
+  return (int32_t)most;
 }
 
 namespace {
@@ -83,6 +110,9 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
     throw Error("groupBytes must not exceed 256 bytes per lane of the block (group prefetch registers)");
   if (plan.groupBytes < 1024 || plan.groupBytes > 65536) throw Error("groupBytes must be in [1024, 65536]");
 
+  if (plan.quantizedRows && (plan.kernel != LaunchPlan::Kernel::kRowParallelLds || plan.rowsPerBlock != 64))
+    throw Error("rank-quantised rows need the row-parallel kernel with 64 rows per block");
+
   PackedModel pm;
   pm.plan = plan;
   pm.numFeatures = forest.numFeatures;
@@ -93,6 +123,28 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
     throw Error("feature offsets do not fit 16 bits for this rowsPerBlock / feature count");
   const uint32_t featureStride = plan.FeatureStride();
   const uint32_t groupCapacity = (uint32_t)plan.groupBytes / kNodeBytes;
+
+  // Rank quantisation: x < t_j  <=>  #{t : t <= x} <= j for the sorted distinct thresholds t_0 < t_1 < ...
+  // of the feature, so an internal node stores j and the kernel compares the row's one-byte rank with it.
+  std::vector<std::vector<float>> ranks;
+  if (plan.quantizedRows) {
+    ranks = ThresholdsPerFeature(forest);
+    size_t most = 0;
+    for (auto &v : ranks) most = std::max(most, v.size());
+    if (most > 254) throw Error("a feature has more than 254 distinct thresholds: rows cannot be rank-quantised to bytes");
+    int32_t depth = 1;
+    while ((size_t)depth < most) depth = depth * 2 + 1; // 2^n - 1 >= most
+    pm.binTableDepth = depth;
+    int32_t chunk = 256;
+    while (chunk > 64 && (int64_t)chunk * depth * 4 > 144 * 1024) chunk /= 2;
+    if ((int64_t)chunk * depth * 4 > 144 * 1024) throw Error("threshold table does not fit LDS");
+    pm.binChunkFeatures = chunk;
+    const int32_t chunks = (forest.numFeatures + chunk - 1) / chunk;
+    pm.binThresholds.assign((size_t)chunks * depth * chunk, std::numeric_limits<float>::quiet_NaN());
+    for (int32_t f = 0; f < forest.numFeatures; ++f)
+      for (size_t k = 0; k < ranks[f].size(); ++k)
+        pm.binThresholds[((size_t)(f / chunk) * depth + k) * chunk + (f % chunk)] = ranks[f][k];
+  }
 
   // Order: class, then depth (the reference sorts by depth for its GPU schedules,
   // src/mlir/GPUAutoSchedule.cpp:115-122); stable so equal keys keep model order.
@@ -174,6 +226,12 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
           const int32_t n = lo.order[i];
           DeviceNode dn;
           dn.value = tree.value[n];
+          if (plan.quantizedRows && !tree.IsLeaf(n)) {
+            const auto &sorted = ranks[(size_t)tree.feature[n]];
+            const uint32_t j = (uint32_t)(std::lower_bound(sorted.begin(), sorted.end(), tree.value[n]) - sorted.begin());
+            static_assert(sizeof(float) == sizeof(uint32_t), "node value holds the rank bit pattern");
+            std::memcpy(&dn.value, &j, sizeof(j));
+          }
           if (tree.IsLeaf(n)) {
             dn.meta = (((base + (uint32_t)i) * kNodeBytes) << 16) | (uint32_t)padOffset;
           } else {
@@ -237,6 +295,13 @@ Tree UnpackTree(const PackedModel &pm, int32_t treeIndex) {
           const int32_t me = pm.nodeOrigin[g.nodeBegin + q];
           const uint32_t child = (dn.meta >> 16) / kNodeBytes;
           tree.value[me] = dn.value;
+          if (child != q && pm.plan.quantizedRows) { // rank -> threshold through the binning table
+            uint32_t j;
+            std::memcpy(&j, &dn.value, sizeof(j));
+            const int32_t f = (int32_t)((dn.meta & 0xFFFFu) / featureStride);
+            const int32_t chunk = pm.binChunkFeatures;
+            tree.value[me] = pm.binThresholds[((size_t)(f / chunk) * pm.binTableDepth + j) * chunk + (f % chunk)];
+          }
           if (child != q) {
             tree.feature[me] = (int32_t)((dn.meta & 0xFFFFu) / featureStride);
             tree.left[me] = pm.nodeOrigin[g.nodeBegin + child];

@@ -27,6 +27,10 @@ struct LaunchPlan {
   int32_t groupBytes = 48 * 1024; // LDS bytes for one tree group's nodes (<= 65536)
   int32_t treeSlices = 1;       // grid.y: how many blocks share one row block's trees
   bool featureOffsetInWords = false;
+  // Row-parallel kernel on rank-quantised rows: a separate kernel first replaces every feature value
+  // by the number of that feature's split thresholds that are <= it (one byte), which preserves the
+  // outcome of every comparison; 64 rows of 1 byte per feature then fit LDS where 64 f32 rows do not.
+  bool quantizedRows = false;
 
   int32_t ThreadsPerBlock() const {
     return kernel == Kernel::kTreeParallel ? rowsPerBlock * treeLanes : rowsPerBlock * treeThreads;
@@ -34,6 +38,7 @@ struct LaunchPlan {
   // Distance in LDS between feature f and f+1 of one row, in the units node offsets use.
   uint32_t FeatureStride() const {
     if (kernel == Kernel::kTreeParallel) return 4u;
+    if (quantizedRows) return (uint32_t)rowsPerBlock / 4u; // byte tile, offsets in units of 4 bytes
     return featureOffsetInWords ? (uint32_t)rowsPerBlock : (uint32_t)rowsPerBlock * 4u;
   }
 };
@@ -50,6 +55,12 @@ struct PackedModel {
   std::vector<int32_t> nodeOrigin; // per packed node: original node id inside its tree (-1: null leaf)
   std::vector<int32_t> slotTree;   // per bundle slot: original tree index, -1 for a padding tree
   uint32_t maxGroupNodes = 0;
+  // Rank quantisation (plan.quantizedRows): per feature the sorted distinct thresholds, stored for the
+  // binning kernel as [featureChunk][k][binChunkFeatures] with NaN behind a feature's last threshold;
+  // binTableDepth = 2^n - 1 entries per feature.
+  std::vector<float> binThresholds;
+  int32_t binTableDepth = 0;
+  int32_t binChunkFeatures = 0;
 
   uint32_t PadFeatureOffset() const;
   // LDS bytes of the tree-group region (regressors reuse it for the tree threads' cross-wave pass).
@@ -64,6 +75,9 @@ struct PackedModel {
   size_t RowTileBytes() const;
   size_t LdsBytes() const; // row tile + the largest group (+ reduction scratch)
 };
+
+// Largest number of distinct split thresholds any one feature has (after comparison normalisation).
+int32_t MaxThresholdsPerFeature(const Forest &forest);
 
 // Throws tbamd::Error when the plan cannot hold the model (tree larger than a
 // group, feature offsets that do not fit 16 bits, ...).

@@ -53,6 +53,7 @@ InferenceRunner::~InferenceRunner() {
   if (m_stream) (void)hipStreamSynchronize(m_stream);
   FreeModel();
   (void)hipFree(m_dPartial);
+  (void)hipFree(m_dRanks);
   (void)hipFree(m_dStageIn);
   (void)hipFree(m_dStageOut);
   if (m_evStart) (void)hipEventDestroy(m_evStart);
@@ -66,6 +67,8 @@ void InferenceRunner::FreeModel() {
   (void)hipFree(m_dGroups);
   (void)hipFree(m_dNodeOrigin);
   (void)hipFree(m_dSlotTree);
+  (void)hipFree(m_dBinTable);
+  m_dBinTable = nullptr;
   m_dNodes = nullptr;
   m_dBundles = nullptr;
   m_dGroups = nullptr;
@@ -82,6 +85,7 @@ void InferenceRunner::UploadModel() {
   m_dGroups = Upload(m_model.groups, "upload groups");
   m_dNodeOrigin = Upload(m_model.nodeOrigin, "upload node origins");
   m_dSlotTree = Upload(m_model.slotTree, "upload slot table");
+  if (m_model.plan.quantizedRows) m_dBinTable = Upload(m_model.binThresholds, "upload threshold table");
 }
 
 void InferenceRunner::Repack(const LaunchPlan &plan) {
@@ -104,6 +108,27 @@ void InferenceRunner::EnsurePartial(int64_t rows) {
   m_partialBytes = need;
 }
 
+void InferenceRunner::EnsureRanks(int64_t rows) {
+  if (!m_model.plan.quantizedRows) return;
+  const size_t need = (size_t)((rows + 63) / 64) * 64 * (size_t)m_forest.numFeatures;
+  if (need <= m_ranksBytes) return;
+  Check(hipStreamSynchronize(m_stream), "hipStreamSynchronize");
+  (void)hipFree(m_dRanks);
+  m_dRanks = nullptr;
+  m_ranksBytes = 0;
+  Check(hipMalloc(reinterpret_cast<void **>(&m_dRanks), need), "allocate rank-quantised rows");
+  m_ranksBytes = need;
+}
+
+const float *InferenceRunner::PrepareRows(const float *deviceInputs, int64_t rows) {
+  if (!m_model.plan.quantizedRows) return deviceInputs;
+  EnsureRanks(rows);
+  Check(LaunchBinRows(deviceInputs, m_dBinTable, m_dRanks, rows, m_forest.numFeatures, m_model.binTableDepth,
+                      m_model.binChunkFeatures, m_stream),
+        "launch rank-quantisation kernel");
+  return reinterpret_cast<const float *>(m_dRanks);
+}
+
 void InferenceRunner::EnsureStaging() {
   if (m_dStageIn) return;
   const size_t rows = (size_t)m_options.batchSize;
@@ -115,7 +140,8 @@ hipError_t InferenceRunner::LaunchWalk(const WalkParams &p) const {
   const LaunchPlan &plan = m_model.plan;
   if (plan.kernel == LaunchPlan::Kernel::kTreeParallel)
     return LaunchWalkTreeParallel(p, plan.interleave, m_model.LdsBytes(), m_stream);
-  return LaunchWalkRowsLds(p, plan.interleave, plan.featureOffsetInWords, m_model.LdsBytes(), m_stream);
+  const int tileMode = plan.quantizedRows ? 2 : (plan.featureOffsetInWords ? 1 : 0);
+  return LaunchWalkRowsLds(p, plan.interleave, tileMode, m_model.LdsBytes(), m_stream);
 }
 
 WalkParams InferenceRunner::MakeWalkParams(const float *deviceInputs, int64_t rows) const {
@@ -143,7 +169,7 @@ void InferenceRunner::Launch(const float *deviceInputs, int64_t rows, float *out
                              float *probabilities, int32_t *leafIds) {
   if (rows <= 0) return;
   EnsurePartial(rows);
-  WalkParams p = MakeWalkParams(deviceInputs, rows);
+  WalkParams p = MakeWalkParams(PrepareRows(deviceInputs, rows), rows);
   const bool finalize = NeedsFinalize();
   p.out = finalize ? nullptr : out;
   p.partial = finalize ? m_dPartial : nullptr;
@@ -218,18 +244,29 @@ void InferenceRunner::RunInference(const void *hostInputs, void *hostResults) {
 }
 
 void InferenceRunner::TimeKernels(const float *deviceInputs, void *deviceResults, int64_t rows, int32_t runs,
-                                  double *walkMs, double *finalizeMs) {
+                                  double *walkMs, double *finalizeMs, double *binMs) {
   runs = std::max(1, runs);
   EnsurePartial(rows);
   const bool finalize = NeedsFinalize();
-  WalkParams p = MakeWalkParams(deviceInputs, rows);
+  float ms = 0.f;
+  if (binMs) *binMs = 0.0;
+  const float *walkInputs = deviceInputs;
+  if (m_model.plan.quantizedRows) {
+    EnsureRanks(rows);
+    Check(hipEventRecord(m_evStart, m_stream), "hipEventRecord");
+    for (int i = 0; i < runs; ++i) walkInputs = PrepareRows(deviceInputs, rows);
+    Check(hipEventRecord(m_evStop, m_stream), "hipEventRecord");
+    Check(hipStreamSynchronize(m_stream), "rank-quantisation kernel");
+    Check(hipEventElapsedTime(&ms, m_evStart, m_evStop), "hipEventElapsedTime");
+    if (binMs) *binMs = ms / runs;
+  }
+  WalkParams p = MakeWalkParams(walkInputs, rows);
   p.out = finalize ? nullptr : static_cast<float *>(deviceResults);
   p.partial = finalize ? m_dPartial : nullptr;
   Check(hipEventRecord(m_evStart, m_stream), "hipEventRecord");
   for (int i = 0; i < runs; ++i) Check(LaunchWalk(p), "launch walk kernel");
   Check(hipEventRecord(m_evStop, m_stream), "hipEventRecord");
   Check(hipStreamSynchronize(m_stream), "walk kernel");
-  float ms = 0.f;
   Check(hipEventElapsedTime(&ms, m_evStart, m_evStop), "hipEventElapsedTime");
   if (walkMs) *walkMs = ms / runs;
   if (finalizeMs) *finalizeMs = 0.0;
@@ -265,16 +302,16 @@ double InferenceRunner::AutoTune(const float *deviceInputs, int64_t rows) {
       } catch (const Error &) {
         continue; // plan cannot hold this model
       }
-      double w = 0, f = 0;
+      double w = 0, f = 0, b = 0;
       try {
-        TimeKernels(deviceInputs, out, rows, 1, &w, &f); // warm-up
-        TimeKernels(deviceInputs, out, rows, 3, &w, &f);
+        TimeKernels(deviceInputs, out, rows, 1, &w, &f, &b); // warm-up
+        TimeKernels(deviceInputs, out, rows, 3, &w, &f, &b);
       } catch (const Error &) {
         (void)hipGetLastError(); // plan the launcher rejects (e.g. too few lanes to prefetch a group)
         continue;
       }
-      if (w + f < bestMs) {
-        bestMs = w + f;
+      if (w + f + b < bestMs) {
+        bestMs = w + f + b;
         best = m_model.plan;
       }
     }
@@ -294,7 +331,8 @@ std::string InferenceRunner::DescribePlan() const {
      << " rowsPerBlock=" << p.rowsPerBlock << " treeThreads=" << p.treeThreads << " treeLanes=" << p.treeLanes
      << " interleave=" << p.interleave
      << " groupBytes=" << p.groupBytes << " treeSlices=" << p.treeSlices
-     << " offsetsInWords=" << (p.featureOffsetInWords ? 1 : 0) << " groups=" << m_model.groups.size()
+     << " offsetsInWords=" << (p.featureOffsetInWords ? 1 : 0) << " quantizedRows=" << (p.quantizedRows ? 1 : 0)
+     << " groups=" << m_model.groups.size()
      << " bundles=" << m_model.bundles.size() << " nodes=" << m_model.nodes.size()
      << " ldsBytes=" << m_model.LdsBytes();
   return os.str();

@@ -40,11 +40,11 @@ public:
                            float *probabilities);
   // Parity check: original leaf node id reached by every (row, tree), int32[rows][numTrees].
   void DumpLeafIds(const float *deviceInputs, int32_t *deviceLeafIds, int64_t rows);
-  // Average duration in milliseconds of the walk kernel (and of the finalize
-  // kernel when the plan needs one) over `runs` launches, HIP events on the
-  // runner's stream.
+  // Average duration in milliseconds of the walk kernel, of the finalize kernel and of the
+  // rank-quantisation kernel (0 when the plan does not use them) over `runs` launches each,
+  // HIP events on the runner's stream.
   void TimeKernels(const float *deviceInputs, void *deviceResults, int64_t rows, int32_t runs, double *walkMs,
-                   double *finalizeMs);
+                   double *finalizeMs, double *binMs);
   // Re-packs the model for another launch plan (used by the timed search).
   void Repack(const LaunchPlan &plan);
   // Timed search over CandidatePlans(); keeps the fastest.  Returns its time in ms.
@@ -66,6 +66,9 @@ private:
   void FreeModel();
   void EnsurePartial(int64_t rows);
   void EnsureStaging();
+  void EnsureRanks(int64_t rows);
+  // Rank-quantised plans: runs the binning kernel and returns the buffer the walk kernel reads.
+  const float *PrepareRows(const float *deviceInputs, int64_t rows);
   bool NeedsFinalize() const { return m_model.plan.treeSlices > 1 || m_forest.numClasses > 0; }
   WalkParams MakeWalkParams(const float *deviceInputs, int64_t rows) const;
   hipError_t LaunchWalk(const WalkParams &p) const;
@@ -86,6 +89,9 @@ private:
   int32_t *m_dSlotTree = nullptr;
   double *m_dPartial = nullptr;
   size_t m_partialBytes = 0;
+  float *m_dBinTable = nullptr;
+  uint8_t *m_dRanks = nullptr;
+  size_t m_ranksBytes = 0;
   float *m_dStageIn = nullptr;
   void *m_dStageOut = nullptr;
   int64_t m_lastKernelMicros = 0;

@@ -322,8 +322,8 @@ int32_t tbmi_dump_leaf_ids(intptr_t h, const float *in, int32_t *ids, int64_t ro
 }
 
 int32_t tbmi_time_kernels(intptr_t h, const float *in, void *out, int64_t rows, int32_t runs, double *walkMs,
-                          double *finalizeMs) {
-  return Guard([&] { Runner(h)->TimeKernels(in, out, rows, runs, walkMs, finalizeMs); return 0; }, -1);
+                          double *finalizeMs, double *binMs) {
+  return Guard([&] { Runner(h)->TimeKernels(in, out, rows, runs, walkMs, finalizeMs, binMs); return 0; }, -1);
 }
 
 int32_t tbmi_autotune(intptr_t h, const float *in, int64_t rows, double *bestMs) {
@@ -338,6 +338,7 @@ int32_t tbmi_set_plan(intptr_t h, int32_t rowsPerBlock, int32_t treeThreads, int
         LaunchPlan plan = r->Model().plan;
         plan.kernel = LaunchPlan::Kernel::kRowParallelLds;
         plan.treeLanes = 1;
+        plan.quantizedRows = false;
         if (rowsPerBlock > 0) plan.rowsPerBlock = rowsPerBlock;
         plan.treeThreads = treeThreads > 0 ? treeThreads : 1;
         if (interleave > 0) plan.interleave = interleave;
@@ -359,6 +360,7 @@ int32_t tbmi_set_tree_parallel_plan(intptr_t h, int32_t rowsPerBlock, int32_t tr
         LaunchPlan plan = r->Model().plan;
         plan.kernel = LaunchPlan::Kernel::kTreeParallel;
         plan.featureOffsetInWords = false;
+        plan.quantizedRows = false;
         plan.treeThreads = 1;
         plan.rowsPerBlock = rowsPerBlock;
         plan.treeLanes = treeLanes;
@@ -366,6 +368,28 @@ int32_t tbmi_set_tree_parallel_plan(intptr_t h, int32_t rowsPerBlock, int32_t tr
         if (groupBytes > 0) plan.groupBytes = groupBytes;
         else plan.groupBytes = std::min(plan.groupBytes, 256 * plan.ThreadsPerBlock());
         if (treeSlices > 0) plan.treeSlices = treeSlices;
+        r->Repack(plan);
+        return 0;
+      },
+      -1);
+}
+
+int32_t tbmi_set_quantized_plan(intptr_t h, int32_t treeThreads, int32_t interleave, int32_t groupBytes,
+                                int32_t treeSlices) {
+  return Guard(
+      [&] {
+        InferenceRunner *r = Runner(h);
+        LaunchPlan plan = r->Model().plan;
+        plan.kernel = LaunchPlan::Kernel::kRowParallelLds;
+        plan.quantizedRows = true;
+        plan.featureOffsetInWords = false;
+        plan.rowsPerBlock = 64;
+        plan.treeLanes = 1;
+        plan.treeThreads = treeThreads > 0 ? treeThreads : 8;
+        plan.interleave = interleave > 0 ? interleave : 4;
+        if (groupBytes > 0) plan.groupBytes = groupBytes;
+        else plan.groupBytes = std::min(plan.groupBytes, 256 * plan.ThreadsPerBlock());
+        plan.treeSlices = treeSlices > 0 ? treeSlices : 1;
         r->Repack(plan);
         return 0;
       },

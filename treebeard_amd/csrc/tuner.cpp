@@ -83,8 +83,35 @@ LaunchPlan ChoosePlan(const Forest &forest, int64_t batchSize, const GPUAutoSche
     bool words = false;
     fitsTransposed = RowTileFits(forest.numFeatures, 64, limits.ldsBytesPerBlock, &words);
   }
-  if (!fitsTransposed || (batchSize > 0 && batchSize <= 128))
+  if (batchSize > 0 && batchSize <= 128) return ChooseTreeParallelPlan(forest, batchSize, ov, limits);
+  if (!fitsTransposed) {
+    // Rows too wide for 64 f32 rows in LDS: one-byte ranks (exact) if every feature has few enough
+    // distinct thresholds and 64 rank rows fit; otherwise a few f32 rows with several lanes each.
+    const int64_t tile = (int64_t)(forest.numFeatures + 1) * 64;
+    const int64_t need = (BiggestTreeNodes(forest) + 2) * kNodeBytes;
+    const int64_t room = limits.ldsBytesPerBlock - tile - 2048 - (forest.numClasses > 0 ? 1024 * 8 : 0);
+    if (room >= std::max<int64_t>(need, 8192) && forest.numFeatures * 16 <= 0xFFFF &&
+        MaxThresholdsPerFeature(forest) <= 254) {
+      LaunchPlan plan;
+      plan.kernel = LaunchPlan::Kernel::kRowParallelLds;
+      plan.quantizedRows = true;
+      plan.rowsPerBlock = 64;
+      plan.treeThreads = 16;
+      if (ov && ov->numTreeThreads > 0) plan.treeThreads = std::max(1, std::min(ov->numTreeThreads, 16));
+      plan.interleave = 2;
+      if (ov && ov->treeWalkInterleaveFactor > 0)
+        plan.interleave = std::min(kMaxInterleave, FloorPow2(ov->treeWalkInterleaveFactor));
+      plan.groupBytes = (int32_t)(std::min<int64_t>({room, 65536, 256LL * plan.ThreadsPerBlock()}) & ~15);
+      const int64_t rowBlocks = std::max<int64_t>(1, (batchSize + 63) / 64);
+      const int64_t totalBytes = (int64_t)forest.NumNodes() * kNodeBytes;
+      int64_t slices = 1;
+      if (rowBlocks < limits.computeUnits) slices = (limits.computeUnits + rowBlocks - 1) / rowBlocks;
+      slices = std::min<int64_t>(slices, std::max<int64_t>(1, totalBytes / plan.groupBytes));
+      plan.treeSlices = (int32_t)std::max<int64_t>(1, slices);
+      return plan;
+    }
     return ChooseTreeParallelPlan(forest, batchSize, ov, limits);
+  }
 
   LaunchPlan plan;
   plan.kernel = LaunchPlan::Kernel::kRowParallelLds;

@@ -285,10 +285,21 @@ class TreebeardInferenceRunner:
                  "tbmi_dump_leaf_ids")
 
     def time_kernels(self, device_inputs_ptr, device_results_ptr, rows, runs):
-        walk, fin = ctypes.c_double(), ctypes.c_double()
+        """(walk ms, finalize + rank-quantisation ms) per launch."""
+        walk, fin, pre = self.time_kernels3(device_inputs_ptr, device_results_ptr, rows, runs)
+        return walk, fin + pre
+
+    def time_kernels3(self, device_inputs_ptr, device_results_ptr, rows, runs):
+        """(walk ms, finalize ms, rank-quantisation ms) per launch."""
+        walk, fin, pre = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
         self._rc(_lib().tbmi_time_kernels(self.inferenceRunner, device_inputs_ptr, device_results_ptr, rows, runs,
-                                          ctypes.byref(walk), ctypes.byref(fin)), "tbmi_time_kernels")
-        return walk.value, fin.value
+                                          ctypes.byref(walk), ctypes.byref(fin), ctypes.byref(pre)),
+                 "tbmi_time_kernels")
+        return walk.value, fin.value, pre.value
+
+    def set_quantized_plan(self, tree_threads=8, interleave=4, group_bytes=0, tree_slices=1):
+        self._rc(_lib().tbmi_set_quantized_plan(self.inferenceRunner, tree_threads, interleave, group_bytes,
+                                                tree_slices), "tbmi_set_quantized_plan")
 
     def autotune(self, device_inputs_ptr, rows):
         best = ctypes.c_double()
