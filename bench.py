@@ -20,7 +20,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0                      # MI355X HBM3E, published
-LDS_PEAK_GBS = 256 * 128 * 2.4             # 256 CUs x 128 B/clk x 2.4 GHz = 78 643 GB/s, nominal
+LDS_PEAK_GBS = 256 * 256 * 2.4             # 256 CUs x 256 B/clk x 2.4 GHz = 157 286 GB/s, nominal
 
 
 def main():
@@ -73,22 +73,34 @@ def main():
     ms_per_step = elapsed / args.steps * 1e3
     rows_per_s = rows / (elapsed / args.steps)
 
-    # kernel-only duration of the dominant (walk) kernel: HIP events on the stream it is launched on
-    walk_ms, fin_ms = runner.time_kernels(dx.data_ptr(), out.data_ptr(), rows, max(args.steps, 5))
+    # kernel-only durations: HIP events on the stream the kernels are launched on (the runtime's own)
+    walk_ms, fin_ms, bin_ms = runner.time_kernels3(dx.data_ptr(), out.data_ptr(), rows, max(args.steps, 5))
+    path_ms = walk_ms + fin_ms + bin_ms
 
-    # algorithmic bytes per row: HBM = 4 F + output; LDS = visited internal nodes x 6 B + 4 B per leaf,
-    # the visit count measured exactly by the oracle on a sample of the same rows
+    # algorithmic bytes per row.  HBM: the row once (4 F) + the output.  LDS: every visited internal node reads
+    # 6 B of node (f32 threshold + i16 feature index) and the 4 B feature value from the LDS row tile, every tree
+    # ends with a 4 B leaf read; the visit count is measured exactly by the oracle on a sample of the same rows.
     from oracle import cpu_oracle, model_io
     forest = model_io.load_xgboost_json(model)
     sample = min(rows, 8192)
     steps_per_row = cpu_oracle.total_steps(forest, x[:sample]) / sample
     hbm_bytes_row = 4 * cfg.num_features + (1 if multiclass else 4)
-    lds_bytes_row = steps_per_row * 6 + 4 * forest.num_trees
-    hbm_gbs = hbm_bytes_row * rows / (walk_ms * 1e-3) / 1e9
-    lds_gbs = lds_bytes_row * rows / (walk_ms * 1e-3) / 1e9
+    lds_bytes_row = steps_per_row * 10 + 4 * forest.num_trees
     hbm_time = hbm_bytes_row * rows / (HBM_PEAK_GBS * 1e9)
     lds_time = lds_bytes_row * rows / (LDS_PEAK_GBS * 1e9)
     binding = "lds" if lds_time > hbm_time else "hbm"
+    plan = runner.describe_plan()
+    quantized = "quantizedRows=1" in plan
+    kernel = "WalkRowsLdsKernel" if "rows_lds" in plan else "WalkTreeParallelKernel"
+    # the rank-quantised path reads the f32 rows in its binning kernel: both kernels count for the HBM roofline
+    hbm_ms = walk_ms + bin_ms if quantized else walk_ms
+    hbm_gbs = hbm_bytes_row * rows / (hbm_ms * 1e-3) / 1e9
+    lds_gbs = lds_bytes_row * rows / (walk_ms * 1e-3) / 1e9
+    traffic = None
+    traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(traffic_file):
+        with open(traffic_file) as fh:
+            traffic = json.load(fh).get("%s@%d" % (cfg.name, rows), {}).get("bytes_per_launch")
 
     line = {
         "metric": "rows/sec at 1 MI355X (2^20-row batch) + % of binding HBM/LDS roofline",
@@ -96,36 +108,50 @@ def main():
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": cfg.name, "rows": rows, "trees": forest.num_trees, "features": cfg.num_features,
-                   "objective": cfg.objective, "plan": runner.describe_plan()},
+                   "objective": cfg.objective, "plan": plan},
         "roofline": {"bound": "hbm", "achieved": hbm_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": hbm_gbs / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "WalkRowsLdsKernel" if "rows_lds" in runner.describe_plan() else "WalkTreeParallelKernel",
-                     "kernel_ms": walk_ms, "finalize_ms": fin_ms, "algorithmic_bytes_per_row": hbm_bytes_row},
+                     "frac": hbm_gbs / HBM_PEAK_GBS, "traffic": traffic,
+                     "kernel": ("BinRowsKernel+" if quantized else "") + kernel,
+                     "kernel_ms": walk_ms, "finalize_ms": fin_ms, "bin_ms": bin_ms,
+                     "algorithmic_bytes_per_row": hbm_bytes_row},
         "roofline_binding": {"bound": binding, "achieved": lds_gbs if binding == "lds" else hbm_gbs,
                              "peak": LDS_PEAK_GBS if binding == "lds" else HBM_PEAK_GBS, "unit": "GB/s",
                              "frac": (lds_gbs / LDS_PEAK_GBS) if binding == "lds" else (hbm_gbs / HBM_PEAK_GBS),
+                             "kernel": kernel, "kernel_ms": walk_ms, "path_ms": path_ms,
                              "algorithmic_bytes_per_row": lds_bytes_row if binding == "lds" else hbm_bytes_row,
                              "visited_nodes_per_row": steps_per_row,
-                             "peak_note": "nominal LDS bandwidth 256 CUs x 128 B/clk x 2.4 GHz"},
+                             "peak_note": "LDS: 256 CUs x 256 B/clk x 2.4 GHz (ds_read_b128 measured 237 B/clk/CU); "
+                                          "a scalar walk moves 10 B per lane per two LDS instructions (4 clk), so "
+                                          "62.5 % is its ceiling"},
     }
 
     if not args.no_cpu_baseline:
+        # The reference's multithreaded CPU configuration restated in oracle/tiled_oracle.c: uniform tiling with
+        # tile size 8, sparse tile layout + LUT, trees ordered by depth, the batch split evenly over the threads,
+        # one tree at a time inside a chunk, f32 accumulation.  Timed on a bounded sample of the same batch.
         threads = cpu_oracle.max_threads()
         order = np.argsort([forest.depth(t) for t in range(forest.num_trees)], kind="stable").astype(np.int32)
-        probe = min(rows, 2048)
+        if multiclass:
+            run = lambda n: cpu_oracle.predict(forest, x[:n], threads=threads)[0]
+            what = "scalar walk, rows split over %d threads (the tiled schedule has no multiclass form here)" % threads
+        else:
+            tiled = cpu_oracle.TiledForest(forest, 8)
+            run = lambda n: tiled.predict_tree_outer(x[:n], tree_order=order, threads=threads)
+            what = ("uniform tiling, tile size 8, sparse layout + LUT, depth-ordered trees, one tree at a time, "
+                    "batch split over %d threads" % threads)
+        probe = min(rows, 4096)
+        run(probe)
         t0 = time.perf_counter()
-        cpu_oracle.predict_tree_outer(forest, x[:probe], tree_order=order, threads=threads)
+        run(probe)
         per_row = (time.perf_counter() - t0) / probe
         cpu_rows = int(min(rows, max(probe, args.cpu_seconds / max(per_row, 1e-9))))
         t0 = time.perf_counter()
-        cpu_out = cpu_oracle.predict_tree_outer(forest, x[:cpu_rows], tree_order=order, threads=threads)
+        cpu_out = run(cpu_rows)
         cpu_s = time.perf_counter() - t0
         line["cpu_baseline"] = {"value": cpu_rows / cpu_s, "unit": "rows/s", "cores": threads, "kind": "port",
-                                "sample": "first %d rows of the same batch, one-tree-at-a-time schedule, batch split "
-                                          "over %d threads, scalar walk (tile size 1)" % (cpu_rows, threads)}
-        if not multiclass:
-            got = out[:cpu_rows].cpu().numpy()
-            line["cpu_baseline"]["max_abs_diff_vs_gpu"] = float(np.abs(got - cpu_out).max())
+                                "sample": "first %d rows of the same batch; %s" % (cpu_rows, what)}
+        got = out[:cpu_rows].cpu().numpy().astype(np.float32)
+        line["cpu_baseline"]["max_abs_diff_vs_gpu"] = float(np.abs(got - cpu_out).max())
     print(json.dumps(line))
 
 

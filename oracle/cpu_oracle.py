@@ -131,6 +131,69 @@ def predict_tree_outer(forest, x, tree_order=None, threads=0):
 
 
 # --------------------------------------------------------------------------
+# tiled CPU walk (oracle/tiled_oracle.c)
+# --------------------------------------------------------------------------
+class TiledForest:
+    """Uniformly tiled, sparse-layout forest with its LUT (tile size 1..8)."""
+
+    def __init__(self, forest, tile_size):
+        assert forest.predicate == 0, "the tiled walk takes 'x < threshold goes left' forests"
+        L = lib()
+        L.tiled_forest_build.restype = ctypes.c_void_p
+        L.tiled_forest_num_tiles.restype = ctypes.c_int64
+        self._L = L
+        self.forest = forest
+        self.tile_size = tile_size
+        keep = c_forest(forest)[1]
+        self.h = ctypes.c_void_p(L.tiled_forest_build(
+            ctypes.c_int32(forest.num_trees), ctypes.c_int32(forest.num_features), _ptr(keep[0]), _ptr(keep[1]),
+            _ptr(keep[2]), _ptr(keep[3]), _ptr(keep[4]), ctypes.c_int32(tile_size)))
+        assert self.h, "tile size must be in 1..8"
+
+    def __del__(self):
+        try:
+            self._L.tiled_forest_free(self.h)
+        except Exception:
+            pass
+
+    def num_tiles(self):
+        return int(self._L.tiled_forest_num_tiles(self.h))
+
+    def num_shapes(self):
+        return int(self._L.tiled_forest_num_shapes(self.h))
+
+    def shapes_with_nodes(self, n):
+        return int(self._L.tiled_forest_shapes_with_nodes(self.h, ctypes.c_int32(n)))
+
+    def leaf_ids(self, x, threads=0):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        ids = np.empty((x.shape[0], self.forest.num_trees), dtype=np.int32)
+        self._L.tiled_leaf_ids(self.h, _ptr(x), ctypes.c_int64(x.shape[0]), _ptr(ids),
+                               ctypes.c_int32(threads or max_threads()))
+        return ids
+
+    def predict_tree_outer(self, x, tree_order=None, threads=0):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        out = np.empty(x.shape[0], dtype=np.float32)
+        order = None if tree_order is None else np.ascontiguousarray(tree_order, dtype=np.int32)
+        self._L.tiled_predict_tree_outer(self.h, _ptr(x), ctypes.c_int64(x.shape[0]),
+                                         ctypes.c_float(self.forest.initial_value),
+                                         ctypes.c_int32(1 if self.forest.transform == 1 else 0), _ptr(out),
+                                         _ptr(order) if order is not None else None,
+                                         ctypes.c_int32(threads or max_threads()))
+        return out
+
+
+def lut_for_shape(left_slot, right_slot, tile_size):
+    """LUT row (2^tile_size entries) of a tile whose nodes (level order) have the given children slots (-1: exit)."""
+    l = np.ascontiguousarray(left_slot, dtype=np.int32)
+    r = np.ascontiguousarray(right_slot, dtype=np.int32)
+    row = np.empty(1 << tile_size, dtype=np.int8)
+    lib().tiled_lut_for_shape(ctypes.c_int32(len(l)), _ptr(l), _ptr(r), ctypes.c_int32(tile_size), _ptr(row))
+    return row
+
+
+# --------------------------------------------------------------------------
 # oracle/_ref: the reference's own header (DecisionForest.h) behind a C driver
 # --------------------------------------------------------------------------
 _ref = None

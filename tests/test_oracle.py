@@ -181,3 +181,80 @@ def test_tree_outer_schedule_matches_default_within_f32():
     order = np.argsort([forest.depth(t) for t in range(forest.num_trees)], kind="stable").astype(np.int32)
     out = cpu_oracle.predict_tree_outer(forest, x, tree_order=order, threads=3)
     np.testing.assert_allclose(out, pred, rtol=0, atol=1e-6)
+
+
+# --------------------------------------------------------------------------
+# tiled CPU walk (the reference's vectorised CPU path, oracle/tiled_oracle.c)
+# --------------------------------------------------------------------------
+@pytest.mark.parametrize("tile_size", [1, 2, 3, 4, 8])
+def test_tiled_walk_reaches_the_scalar_leaf_on_reference_models(tile_size):
+    paths = random_models()[::4] + [benchmark_model("higgs"), benchmark_model("year_prediction_msd")]
+    for path in paths:
+        forest = model_io.load_xgboost_json(path)
+        csv = path[:-3] + ".csv" if path.endswith(".gz") else path + ".csv"
+        x, _ = model_io.read_csv(csv, max_rows=120)
+        x = x.astype(np.float32)
+        tiled = cpu_oracle.TiledForest(forest, tile_size)
+        np.testing.assert_array_equal(tiled.leaf_ids(x), cpu_oracle.leaf_ids(forest, x))
+
+
+@pytest.mark.parametrize("tile_size", [2, 3, 4, 8])
+def test_tiled_walk_on_random_and_degenerate_trees(tile_size, tmp_path):
+    from treebeard_amd import synth
+    rng = np.random.Generator(np.random.PCG64(tile_size))
+    trees = [synth._grow_tree(rng, 9, lambda d, s: 0.75, lambda: (rng.integers(0, 6), np.round(rng.normal(), 1)),
+                              lambda: rng.normal()) for _ in range(60)]
+    trees.append(synth._grow_tree(rng, 0, lambda d, s: 0.0, lambda: (0, 0.0), lambda: 0.5, force_root=False))  # single leaf
+    trees.append(synth._grow_tree(rng, 10, lambda d, s: 1.0 if s <= 0 else 0.0, lambda: (1, rng.normal()), lambda: rng.normal()))
+    trees.append(synth._grow_tree(rng, 10, lambda d, s: 1.0 if s != 0 else 0.0, lambda: (2, rng.normal()), lambda: rng.normal()))
+    path = tmp_path / "m.json"
+    synth.write_xgboost_json(path, trees, 6)
+    forest = model_io.load_xgboost_json(path)
+    x = np.round(rng.normal(size=(400, 6)), 1).astype(np.float32)     # many values equal to thresholds
+    tiled = cpu_oracle.TiledForest(forest, tile_size)
+    np.testing.assert_array_equal(tiled.leaf_ids(x), cpu_oracle.leaf_ids(forest, x))
+    pred, _ = cpu_oracle.predict(forest, x)
+    np.testing.assert_allclose(tiled.predict_tree_outer(x, threads=3), pred, rtol=1e-5, atol=1e-5)
+
+
+def test_tile_shapes_and_lut_known_answers():
+    import math
+    # left chain of three nodes (docs/TileShapesAndLUT/TileShapesAndLUT.md:36-46): node 0 -> left node 1 -> left node 2;
+    # outcome strings there are written with node 0 first, the kernel word has node 0 in bit 0
+    row = cpu_oracle.lut_for_shape([1, 2, -1], [-1, -1, -1], 3)
+    word = lambda s: sum(int(c) << i for i, c in enumerate(s))
+    assert row[word("110")] == 1 and row[word("111")] == 0
+    assert all(row[word("0" + a + b)] == 3 for a in "01" for b in "01")        # root false: 4th child whatever the rest
+    assert row[word("100")] == 2 and row[word("101")] == 2
+    # complete tile of three nodes reduces to a textbook two-level descent
+    row = cpu_oracle.lut_for_shape([1, -1, -1], [2, -1, -1], 3)
+    for b0 in (0, 1):
+        for b1 in (0, 1):
+            for b2 in (0, 1):
+                expected = (0 if b1 else 1) if b0 else (2 if b2 else 3)
+                assert row[b0 | b1 << 1 | b2 << 2] == expected
+    # number of tile shapes with exactly T nodes that random forests produce never exceeds Catalan(T), and for
+    # small T a large sample hits every one of them (TileShapesAndLUT.md:15-19: 1, 2, 5, 14, ...)
+    from treebeard_amd import synth
+    rng = np.random.Generator(np.random.PCG64(99))
+    trees = [synth._grow_tree(rng, 8, lambda d, s: 0.7, lambda: (rng.integers(0, 4), rng.normal()), lambda: rng.normal())
+             for _ in range(400)]
+    forest = model_io._assemble([(t.value, t.feature, t.left, t.right) for t in trees], num_features=4, initial_value=0.0,
+                                transform=model_io.IDENTITY, num_classes=0, predicate=model_io.PRED_LT,
+                                class_id=np.zeros(400, np.int32))
+    for tile_size in (1, 2, 3, 4, 8):
+        catalan = math.comb(2 * tile_size, tile_size) // (tile_size + 1)
+        found = cpu_oracle.TiledForest(forest, tile_size).shapes_with_nodes(tile_size)
+        assert found <= catalan
+        if tile_size <= 4:
+            assert found == catalan
+
+
+def test_tiled_multithreaded_schedule_matches_scalar_schedule():
+    forest = model_io.load_xgboost_json(benchmark_model("airline"))
+    x, _ = model_io.read_csv(benchmark_csv("airline"))
+    x = x.astype(np.float32)
+    order = np.argsort([forest.depth(t) for t in range(forest.num_trees)], kind="stable").astype(np.int32)
+    scalar = cpu_oracle.predict_tree_outer(forest, x, tree_order=order, threads=2)
+    tiled = cpu_oracle.TiledForest(forest, 8).predict_tree_outer(x, tree_order=order, threads=5)
+    np.testing.assert_array_equal(tiled, scalar)     # same leaves, same f32 summation order
