@@ -362,3 +362,22 @@ def test_row_staging_alignment_and_ragged_tails(tmp_path, rows, features, offset
         out.fill_(float("nan"))
         runner.run_device(flat.data_ptr() + 4 * offset, out.data_ptr(), rows)
         np.testing.assert_allclose(out.cpu().numpy(), expected, rtol=RTOL_SUM, atol=0)
+
+
+@pytest.mark.parametrize("k,rows", [(2, (1 << 18) + 777), (3, 1 << 17), (4, 5000)])
+def test_host_buffer_entry_point_pipelines_large_batches(synth_model, k, rows):
+    """RunInference on host memory copies and computes a large batch in overlapping pieces: same bits as one launch."""
+    x = synth.CONFIGS[k].batch_rows(rows, seed_offset=2)
+    runner = make_runner(synth_model(k), rows)
+    device = gpu_predict(runner, x)
+    host = runner.RunInference(x, resultType=np.int8 if runner.num_classes() > 0 else np.float32)
+    np.testing.assert_array_equal(host, device)
+    forest = model_io.load_xgboost_json(synth_model(k))
+    pick = np.random.default_rng(k).choice(rows, size=2048, replace=False)
+    pred, _ = cpu_oracle.predict(forest, x[pick])
+    if forest.num_classes > 0:
+        np.testing.assert_array_equal(host[pick].astype(np.float32), pred)
+    elif forest.transform == model_io.SIGMOID:
+        np.testing.assert_allclose(host[pick], pred, rtol=0, atol=ATOL_PROB)
+    else:
+        np.testing.assert_allclose(host[pick], pred, rtol=RTOL_SUM, atol=0)

@@ -56,6 +56,9 @@ InferenceRunner::~InferenceRunner() {
   (void)hipFree(m_dRanks);
   (void)hipFree(m_dStageIn);
   (void)hipFree(m_dStageOut);
+  for (auto &ev : m_pieceReady)
+    if (ev) (void)hipEventDestroy(ev);
+  if (m_copyStream) (void)hipStreamDestroy(m_copyStream);
   if (m_evStart) (void)hipEventDestroy(m_evStart);
   if (m_evStop) (void)hipEventDestroy(m_evStop);
   if (m_stream) (void)hipStreamDestroy(m_stream);
@@ -237,10 +240,41 @@ void InferenceRunner::DumpLeafIds(const float *deviceInputs, int32_t *deviceLeaf
 
 void InferenceRunner::RunInference(const void *hostInputs, void *hostResults) {
   EnsureStaging();
-  const size_t rows = (size_t)m_options.batchSize;
-  Check(hipMemcpyAsync(m_dStageIn, hostInputs, rows * m_forest.numFeatures * sizeof(float), hipMemcpyHostToDevice, m_stream), "copy inputs");
-  RunDevice(m_dStageIn, m_dStageOut, (int64_t)rows);
-  Check(hipMemcpy(hostResults, m_dStageOut, rows * ReturnTypeBytes(), hipMemcpyDeviceToHost), "copy results");
+  const int64_t rows = m_options.batchSize;
+  const size_t rowBytes = (size_t)m_forest.numFeatures * sizeof(float);
+  const bool multiclass = m_forest.numClasses > 0;
+  // Large batches go through in pieces: the copy of piece i+1 (on its own stream) overlaps the kernels
+  // of piece i.  Rows are independent, so the pieces give the same results as one launch.
+  constexpr int kMaxPieces = 8;
+  int pieces = 1;
+  if (!gMeasureGpuKernelTime && (size_t)rows * rowBytes >= ((size_t)16 << 20))
+    pieces = (int)std::min<int64_t>(kMaxPieces, rows / 4096);
+  if (pieces <= 1) {
+    Check(hipMemcpyAsync(m_dStageIn, hostInputs, (size_t)rows * rowBytes, hipMemcpyHostToDevice, m_stream), "copy inputs");
+    RunDevice(m_dStageIn, m_dStageOut, rows);
+  } else {
+    if (!m_copyStream) {
+      Check(hipStreamCreateWithFlags(&m_copyStream, hipStreamNonBlocking), "hipStreamCreate");
+      for (auto &ev : m_pieceReady) Check(hipEventCreateWithFlags(&ev, hipEventDisableTiming), "hipEventCreate");
+    }
+    const int64_t perPiece = ((rows + pieces - 1) / pieces + 1023) / 1024 * 1024;
+    int p = 0;
+    for (int64_t first = 0; first < rows; first += perPiece, ++p) {
+      const int64_t count = std::min(perPiece, rows - first);
+      float *dIn = m_dStageIn + first * m_forest.numFeatures;
+      Check(hipMemcpyAsync(dIn, static_cast<const char *>(hostInputs) + (size_t)first * rowBytes, (size_t)count * rowBytes,
+                           hipMemcpyHostToDevice, m_copyStream),
+            "copy inputs");
+      Check(hipEventRecord(m_pieceReady[p], m_copyStream), "hipEventRecord");
+      Check(hipStreamWaitEvent(m_stream, m_pieceReady[p], 0), "hipStreamWaitEvent");
+      if (multiclass)
+        Launch(dIn, count, nullptr, static_cast<int8_t *>(m_dStageOut) + first, nullptr, nullptr, nullptr);
+      else
+        Launch(dIn, count, static_cast<float *>(m_dStageOut) + first, nullptr, nullptr, nullptr, nullptr);
+    }
+    Check(hipStreamSynchronize(m_stream), "inference kernels");
+  }
+  Check(hipMemcpy(hostResults, m_dStageOut, (size_t)rows * ReturnTypeBytes(), hipMemcpyDeviceToHost), "copy results");
 }
 
 void InferenceRunner::TimeKernels(const float *deviceInputs, void *deviceResults, int64_t rows, int32_t runs,

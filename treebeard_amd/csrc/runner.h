@@ -80,6 +80,8 @@ private:
   DeviceLimits m_limits;
   PackedModel m_model;
   hipStream_t m_stream = nullptr;
+  hipStream_t m_copyStream = nullptr; // host-buffer entry point: copies of the next piece overlap the kernels
+  hipEvent_t m_pieceReady[8] = {};
   hipEvent_t m_evStart = nullptr, m_evStop = nullptr;
 
   DeviceNode *m_dNodes = nullptr;
