@@ -140,6 +140,11 @@ TBAMD_EXPORT int32_t tbmi_set_tree_parallel_plan(intptr_t runner, int32_t rowsPe
 TBAMD_EXPORT int32_t tbmi_set_quantized_plan(intptr_t runner, int32_t treeThreads, int32_t interleave,
                                              int32_t groupBytes, int32_t treeSlices);
 TBAMD_EXPORT int32_t tbmi_describe_plan(intptr_t runner, char *buffer, int32_t length);
+/* Compile once, reload: saves the compiled model (forest + launch plan) of a runner to one file and
+ * reopens it without the source model (batchSize <= 0 keeps the saved batch size).  Stands in for
+ * InitializeInferenceRunner(soPath, globalsJSON), runtime.cpp:35-54. */
+TBAMD_EXPORT int32_t tbmi_save_compiled_model(intptr_t runner, const char *path);
+TBAMD_EXPORT intptr_t tbmi_load_compiled_model(const char *path, int32_t batchSize);
 TBAMD_EXPORT int32_t tbmi_num_trees(intptr_t runner);
 TBAMD_EXPORT int32_t tbmi_num_classes(intptr_t runner);
 
@@ -151,6 +156,11 @@ TBAMD_EXPORT int32_t tbmi_forest_info(intptr_t forest, int64_t *info, double *in
 TBAMD_EXPORT int32_t tbmi_forest_tree_size(intptr_t forest, int32_t tree);
 TBAMD_EXPORT int32_t tbmi_forest_tree(intptr_t forest, int32_t tree, float *value, int32_t *feature, int32_t *left,
                                       int32_t *right, int32_t *classId);
+/* Reads a leaf hit-count profile (the reference's probability profile: `numTrees, numRows`, then per tree
+ * `hitCount, depth` for every leaf in node order) and checks it against the forest; returns the row count
+ * and the average number of internal nodes a profiled row visits. */
+TBAMD_EXPORT int32_t tbmi_forest_load_profile(intptr_t forest, const char *profileCSVPath, int64_t *numRows,
+                                              double *expectedSteps);
 /* Packs the forest for the given plan and unpacks it again; returns the number of trees that differ
  * from the (comparison-normalised) input, or -1 when the plan cannot hold the model.
  * stats[0..4] = groups, bundles, nodes, ldsBytes, paddingTrees. */

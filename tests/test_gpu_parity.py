@@ -381,3 +381,27 @@ def test_host_buffer_entry_point_pipelines_large_batches(synth_model, k, rows):
         np.testing.assert_allclose(host[pick], pred, rtol=0, atol=ATOL_PROB)
     else:
         np.testing.assert_allclose(host[pick], pred, rtol=RTOL_SUM, atol=0)
+
+
+@pytest.mark.parametrize("k", [2, 3, 4])
+def test_compiled_model_file_round_trip(synth_model, tmp_path, k):
+    """Compile once, reload: the saved file reopens without the source model and predicts the same bits."""
+    rows = 2000
+    x = synth.CONFIGS[k].batch_rows(rows, seed_offset=4)
+    runner = make_runner(synth_model(k), rows)
+    if k == 2:
+        runner.set_plan(128, 8, 2, 32768, 3)
+    expected = gpu_predict(runner, x)
+    path = str(tmp_path / "model.tbamd")
+    runner.save_compiled_model(path)
+    plan = runner.describe_plan()
+    del runner
+    reopened = treebeard.TreebeardInferenceRunner.FromCompiledModelFile(path)
+    assert reopened.batchSize == rows and reopened.describe_plan() == plan
+    np.testing.assert_array_equal(gpu_predict(reopened, x), expected)
+    forest = model_io.load_xgboost_json(synth_model(k))
+    np.testing.assert_array_equal(gpu_leaf_ids(reopened, x[:256]), cpu_oracle.leaf_ids(forest, x[:256]))
+    with open(path, "r+b") as fh:
+        fh.truncate(os.path.getsize(path) // 2)
+    with pytest.raises(RuntimeError, match="truncated"):
+        treebeard.TreebeardInferenceRunner.FromCompiledModelFile(path)

@@ -191,3 +191,39 @@ def test_synthetic_configurations_have_the_stated_shape(synth_model):
     assert (f5.num_trees, f5.num_features) == (800, 90) and max(f5.depth(t) for t in range(800)) == 12
     x3 = synth.CONFIGS[3].batch_rows(2000)
     assert set(np.unique(x3[:, 10:])) <= {0.0, 1.0} and 0.05 < x3[:, 10:].mean() < 0.15
+
+
+def test_hit_count_profile_of_the_reference_matches_its_model(lib, plain_file):
+    """xgb_models/profiles/higgs.test.csv against higgs_xgb_model_save.json: per tree the leaf hits add up to numRows."""
+    h = load_forest(lib, plain_file(benchmark_model("higgs")))
+    rows, steps = ctypes.c_int64(), ctypes.c_double()
+    profile = plain_file(os.path.join(GOLDEN, "benchmark", "higgs.test.profile.csv.gz"))
+    assert lib.tbmi_forest_load_profile(h, profile.encode(), ctypes.byref(rows), ctypes.byref(steps)) == 0, last_error()
+    assert rows.value > 1000 and 100 * 1.0 < steps.value <= 100 * 8.0     # 100 trees, depth <= 8
+    lib.tbmi_delete_forest(h)
+    # a profile of another model is refused
+    h = load_forest(lib, plain_file(benchmark_model("airline")))
+    assert lib.tbmi_forest_load_profile(h, profile.encode(), ctypes.byref(rows), ctypes.byref(steps)) == -1
+    assert "hit-count profile" in last_error()
+    lib.tbmi_delete_forest(h)
+
+
+def test_hit_count_profile_agrees_with_oracle_walks(lib, tmp_path, synth_model):
+    """A profile written from the oracle's leaf ids in the reference's format reads back with the oracle's step count."""
+    from oracle import cpu_oracle
+    forest = model_io.load_xgboost_json(synth_model(1))
+    x = synth.CONFIGS[1].batch_rows(500)
+    ids, plen = cpu_oracle.leaf_ids(forest, x, want_path_len=True)
+    lines = ["%d, %d" % (forest.num_trees, x.shape[0])]
+    for t in range(forest.num_trees):
+        _, _, left, _ = forest.tree(t)
+        leaves = np.nonzero(left == -1)[0]
+        hits = [(int((ids[:, t] == leaf).sum()), 6) for leaf in leaves]
+        lines.append(", ".join("%d, %d" % hd for hd in hits))
+    path = tmp_path / "profile.csv"
+    path.write_text("\n".join(lines) + "\n")
+    h = load_forest(lib, synth_model(1))
+    rows, steps = ctypes.c_int64(), ctypes.c_double()
+    assert lib.tbmi_forest_load_profile(h, str(path).encode(), ctypes.byref(rows), ctypes.byref(steps)) == 0, last_error()
+    assert rows.value == 500 and abs(steps.value - plen.sum() / 500) < 1e-9
+    lib.tbmi_delete_forest(h)

@@ -27,6 +27,19 @@ template <typename T> T *Upload(const std::vector<T> &host, const char *what) {
 InferenceRunner::InferenceRunner(Forest forest, const CompilerOptions &options,
                                  const GPUAutoScheduleOptions *gpuOptions)
     : m_forest(std::move(forest)), m_options(options) {
+  InitDevice();
+  m_model = PackForest(m_forest, ChoosePlan(m_forest, m_options.batchSize, gpuOptions, m_limits));
+  UploadModel();
+}
+
+InferenceRunner::InferenceRunner(Forest forest, const CompilerOptions &options, const LaunchPlan &plan)
+    : m_forest(std::move(forest)), m_options(options) {
+  InitDevice();
+  m_model = PackForest(m_forest, plan);
+  UploadModel();
+}
+
+void InferenceRunner::InitDevice() {
   if (m_options.batchSize <= 0) throw Error("batchSize must be positive");
   if (m_options.inputElementTypeWidth != 32) throw Error("only 32-bit float inputs are supported");
   if (m_options.thresholdTypeWidth != 32) throw Error("only 32-bit float thresholds are supported");
@@ -44,9 +57,6 @@ InferenceRunner::InferenceRunner(Forest forest, const CompilerOptions &options,
   Check(hipStreamCreateWithFlags(&m_stream, hipStreamNonBlocking), "hipStreamCreate");
   Check(hipEventCreate(&m_evStart), "hipEventCreate");
   Check(hipEventCreate(&m_evStop), "hipEventCreate");
-
-  m_model = PackForest(m_forest, ChoosePlan(m_forest, m_options.batchSize, gpuOptions, m_limits));
-  UploadModel();
 }
 
 InferenceRunner::~InferenceRunner() {

@@ -27,6 +27,8 @@ extern int32_t gNumberOfKernelRuns;
 class InferenceRunner {
 public:
   InferenceRunner(Forest forest, const CompilerOptions &options, const GPUAutoScheduleOptions *gpuOptions);
+  // Reopens a compiled model: the plan is taken as saved instead of asking the tuner.
+  InferenceRunner(Forest forest, const CompilerOptions &options, const LaunchPlan &plan);
   ~InferenceRunner();
   InferenceRunner(const InferenceRunner &) = delete;
   InferenceRunner &operator=(const InferenceRunner &) = delete;
@@ -62,6 +64,7 @@ public:
   hipStream_t Stream() const { return m_stream; }
 
 private:
+  void InitDevice();
   void UploadModel();
   void FreeModel();
   void EnsurePartial(int64_t rows);

@@ -1,6 +1,7 @@
 // extern "C" surface (include/tbruntime_amd.h).  Nothing throws across it.
 #include "../../include/tbruntime_amd.h"
 
+#include "model_file.h"
 #include "runner.h"
 
 #include <cstring>
@@ -187,7 +188,12 @@ intptr_t CreateInferenceRunner(const char *modelJSONPath, const char *profileCSV
       [&]() -> intptr_t {
         CompilerOptions opts = *Opts(options);
         if (profileCSVPath && *profileCSVPath) opts.statsProfileCSVPath = profileCSVPath;
-        return reinterpret_cast<intptr_t>(new InferenceRunner(LoadXGBoostJSON(modelJSONPath), opts, nullptr));
+        Forest forest = LoadXGBoostJSON(modelJSONPath);
+        // A hit-count profile is checked against the model; the lock-step kernels have no
+        // data-dependent layout, so it does not change the packed model.
+        if (!opts.statsProfileCSVPath.empty() && opts.tilingType != TilingType::kUniform)
+          (void)LoadHitCountProfile(forest, opts.statsProfileCSVPath);
+        return reinterpret_cast<intptr_t>(new InferenceRunner(std::move(forest), opts, nullptr));
       },
       0);
 }
@@ -405,6 +411,43 @@ int32_t tbmi_describe_plan(intptr_t h, char *buffer, int32_t length) {
           buffer[length - 1] = 0;
         }
         return (int32_t)s.size();
+      },
+      -1);
+}
+
+int32_t tbmi_save_compiled_model(intptr_t h, const char *path) {
+  return Guard(
+      [&] {
+        InferenceRunner *r = Runner(h);
+        SaveCompiledModel(path ? path : "", r->GetForest(), r->Model().plan, r->BatchSize());
+        return 0;
+      },
+      -1);
+}
+
+intptr_t tbmi_load_compiled_model(const char *path, int32_t batchSize) {
+  return Guard(
+      [&]() -> intptr_t {
+        CompiledModel m = LoadCompiledModel(path ? path : "");
+        CompilerOptions options;
+        options.batchSize = batchSize > 0 ? batchSize : m.batchSize;
+        return reinterpret_cast<intptr_t>(new InferenceRunner(std::move(m.forest), options, m.plan));
+      },
+      0);
+}
+
+int32_t tbmi_forest_load_profile(intptr_t h, const char *profileCSVPath, int64_t *numRows, double *expectedSteps) {
+  return Guard(
+      [&] {
+        if (!h) throw Error("null forest handle");
+        const Forest *f = reinterpret_cast<const Forest *>(h);
+        HitCountProfile profile = LoadHitCountProfile(*f, profileCSVPath ? profileCSVPath : "");
+        for (size_t t = 0; t < f->trees.size(); ++t)
+          if (profile.hits[t][0] != profile.numRows)
+            throw Error("hit-count profile: the leaf hits of tree " + std::to_string(t) + " do not add up to numRows");
+        if (numRows) *numRows = profile.numRows;
+        if (expectedSteps) *expectedSteps = ExpectedWalkSteps(*f, profile);
+        return 0;
       },
       -1);
 }

@@ -62,6 +62,9 @@ SIGNATURES = {
     "tbmi_set_plan": (c_i32, [c_ip, c_i32, c_i32, c_i32, c_i32, c_i32]),
     "tbmi_set_tree_parallel_plan": (c_i32, [c_ip, c_i32, c_i32, c_i32, c_i32, c_i32]),
     "tbmi_describe_plan": (c_i32, [c_ip, c_cp, c_i32]),
+    "tbmi_save_compiled_model": (c_i32, [c_ip, c_cp]),
+    "tbmi_load_compiled_model": (c_ip, [c_cp, c_i32]),
+    "tbmi_forest_load_profile": (c_i32, [c_ip, c_cp, ctypes.POINTER(c_i64), ctypes.POINTER(ctypes.c_double)]),
     "tbmi_num_trees": (c_i32, [c_ip]),
     "tbmi_num_classes": (c_i32, [c_ip]),
     "tbmi_load_forest": (c_ip, [c_cp, c_cp, c_i32]),

@@ -215,6 +215,15 @@ class TreebeardInferenceRunner:
             onnx_model_path.encode("ascii"), options.optionsPtr), "CreateInferenceRunnerForONNXModel"))
 
     @classmethod
+    def FromCompiledModelFile(cls, path, batchSize=0):
+        """Reopens a model saved with save_compiled_model (the counterpart of the reference's FromSOFile)."""
+        return cls._from_handle(_check(_lib().tbmi_load_compiled_model(path.encode("ascii"), batchSize),
+                                       "tbmi_load_compiled_model"))
+
+    def save_compiled_model(self, path):
+        self._rc(_lib().tbmi_save_compiled_model(self.inferenceRunner, path.encode("ascii")), "tbmi_save_compiled_model")
+
+    @classmethod
     def FromTBContext(cls, tbContext):
         return tbContext.ConstructInferenceRunnerFromHIR()
 
