@@ -145,8 +145,8 @@ LaunchPlan ChoosePlan(const Forest &forest, int64_t batchSize, const GPUAutoSche
   if (need > 65536) throw Error("a tree does not fit one LDS tree group");
   const int64_t meet = forest.numClasses > 0 ? (int64_t)rb * plan.treeThreads * 8 : 0; // cross-wave pass
   // (LDS is handed out in coarse pieces: leave slack or the second block will not fit)
-  int64_t group = std::min<int64_t>(65536, budget - rowTile - meet - 2048);
-  if (group < need) group = std::min<int64_t>(65536, limits.ldsBytesPerBlock - rowTile - meet - 2048);
+  int64_t group = std::min<int64_t>(65536, budget - rowTile - meet - 512);
+  if (group < need) group = std::min<int64_t>(65536, limits.ldsBytesPerBlock - rowTile - meet - 512);
   group = std::min<int64_t>(group, 256LL * rb * plan.treeThreads); // 16 prefetch registers of 16 bytes per lane
   if (group < need) throw Error("the biggest tree does not fit LDS next to the row tile");
   plan.groupBytes = (int32_t)(group & ~15);
