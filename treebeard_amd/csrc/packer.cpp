@@ -135,8 +135,9 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
     int32_t depth = 1;
     while ((size_t)depth < most) depth = depth * 2 + 1; // 2^n - 1 >= most
     pm.binTableDepth = depth;
+    // features per block of the binning kernel: two blocks per CU when the table allows it
     int32_t chunk = 256;
-    while (chunk > 64 && (int64_t)chunk * depth * 4 > 144 * 1024) chunk /= 2;
+    while (chunk > 64 && (int64_t)chunk * depth * 4 > 72 * 1024) chunk /= 2;
     if ((int64_t)chunk * depth * 4 > 144 * 1024) throw Error("threshold table does not fit LDS");
     pm.binChunkFeatures = chunk;
     const int32_t chunks = (forest.numFeatures + chunk - 1) / chunk;
