@@ -405,3 +405,38 @@ def test_compiled_model_file_round_trip(synth_model, tmp_path, k):
         fh.truncate(os.path.getsize(path) // 2)
     with pytest.raises(RuntimeError, match="truncated"):
         treebeard.TreebeardInferenceRunner.FromCompiledModelFile(path)
+
+
+@pytest.mark.parametrize("paths", ["default", "rows_lds", "tree_parallel", "quantised"])
+def test_nan_inputs_follow_the_scalar_walk(tmp_path, paths):
+    """NaN compares false, so a NaN feature sends the row to the right child (src/include/DecisionForest.h:372-375)."""
+    path = str(tmp_path / "coarse.json")
+    coarse_model(path, 9, 40, 0, seed=23)
+    forest = model_io.load_xgboost_json(path)
+    rng = np.random.default_rng(8)
+    x = np.round(rng.normal(size=(300, 9)), 2).astype(np.float32)
+    x[rng.random(x.shape) < 0.2] = np.nan
+    runner = make_runner(path, 300)
+    if paths == "rows_lds":
+        runner.set_plan(64, 2, 2, 16384, 2)
+    elif paths == "tree_parallel":
+        runner.set_tree_parallel_plan(4, 16, 1, 16384, 3)
+    elif paths == "quantised":
+        runner.set_quantized_plan(4, 2, 16384, 1)
+    check_against_oracle(runner, forest, x)
+
+
+@pytest.mark.parametrize("k,rows,slices", [(2, 3, 40), (3, 50, 24), (1, 700, 20)])
+def test_many_tree_slices_on_small_batches(synth_model, k, rows, slices):
+    """Few rows spread over many tree slices: the wave-per-row finalize adds the slices."""
+    forest = model_io.load_xgboost_json(synth_model(k))
+    x = synth.CONFIGS[k].batch_rows(rows, seed_offset=6)
+    runner = make_runner(synth_model(k), rows)
+    runner.set_plan(64, 2, 1, 4096 if k != 5 else 16384, slices)
+    assert "treeSlices=%d" % slices in runner.describe_plan()
+    check_against_oracle(runner, forest, x)
+    if k == 3:
+        dx = torch.from_numpy(x).cuda()
+        margins = torch.zeros((rows, 8), dtype=torch.float32, device="cuda")
+        runner.run_device_multiclass(dx.data_ptr(), rows, None, margins.data_ptr(), None)
+        np.testing.assert_allclose(margins.cpu().numpy(), cpu_oracle.predict(forest, x)[1], rtol=RTOL_SUM, atol=1e-7)

@@ -564,6 +564,29 @@ __global__ void __launch_bounds__(256) FinalizeKernel(const FinalizeParams p) {
   }
 }
 
+// Small batches split over many tree slices: one wave per (row, class).  The lanes fetch the slice
+// partials side by side (one memory latency instead of one per slice), each adds its slices in slice
+// order, and a fixed butterfly combines the lanes - the order of additions depends only on the number
+// of slices.
+__global__ void __launch_bounds__(256) FinalizeWideKernel(const FinalizeParams p) {
+  const int lane = threadIdx.x & 63;
+  const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int Cn = p.numClasses > 0 ? p.numClasses : 1;
+  if (item >= p.rows * Cn) return; // (whole waves leave together)
+  const int64_t row = item / Cn;
+  const int c = (int)(item - row * Cn);
+  double sum = 0.0;
+  for (int s = lane; s < p.treeSlices; s += 64) sum += p.partial[((int64_t)s * p.rows + row) * Cn + c];
+  for (int m = 32; m >= 1; m >>= 1) sum += ShuffleXor(sum, m);
+  const double margin = p.initialValue + sum;
+  if (p.numClasses == 0) {
+    if (lane == 0) p.out[row] = (float)(p.transform == 1 ? 1.0 / (1.0 + exp(-margin)) : margin);
+    return;
+  }
+  // classifiers: park the class sum in the first slice's slot; FinalizeKernel (1 slice) does the rest
+  if (lane == 0) const_cast<double *>(p.partial)[row * Cn + c] = margin - p.initialValue;
+}
+
 template <int K, int PF, int W>
 hipError_t LaunchWalkKP(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
   if (p.leafIds) {
@@ -694,8 +717,17 @@ hipError_t LaunchBinRows(const float *x, const float *table, uint8_t *ranks, int
 
 hipError_t LaunchFinalize(const FinalizeParams &p, hipStream_t stream) {
   if (p.rows <= 0) return hipSuccess;
-  const int64_t blocks = (p.rows + 255) / 256;
-  FinalizeKernel<<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(p);
+  const int Cn = p.numClasses > 0 ? p.numClasses : 1;
+  FinalizeParams q = p;
+  if (p.treeSlices >= 16 && p.rows * Cn <= 65536) { // few rows, many slices: a wave per (row, class)
+    const int64_t waves = p.rows * Cn;
+    FinalizeWideKernel<<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream>>>(p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || p.numClasses == 0) return e;
+    q.treeSlices = 1; // the class sums now sit in slice 0
+  }
+  const int64_t blocks = (q.rows + 255) / 256;
+  FinalizeKernel<<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(q);
   return hipGetLastError();
 }
 
