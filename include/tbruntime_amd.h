@@ -136,6 +136,9 @@ TBAMD_EXPORT int32_t tbmi_set_plan(intptr_t runner, int32_t rowsPerBlock, int32_
 /* Pins the tree-parallel kernel: rowsPerBlock rows per block, treeLanes lanes per row. */
 TBAMD_EXPORT int32_t tbmi_set_tree_parallel_plan(intptr_t runner, int32_t rowsPerBlock, int32_t treeLanes,
                                                  int32_t interleave, int32_t groupBytes, int32_t treeSlices);
+/* Pins the global-memory walk (the fallback for trees too big for LDS): one lane per row. */
+TBAMD_EXPORT int32_t tbmi_set_global_walk_plan(intptr_t runner, int32_t rowsPerBlock, int32_t interleave,
+                                               int32_t treeSlices);
 /* Pins the row-parallel kernel on rank-quantised rows (64 rows per block, one byte per feature value). */
 TBAMD_EXPORT int32_t tbmi_set_quantized_plan(intptr_t runner, int32_t treeThreads, int32_t interleave,
                                              int32_t groupBytes, int32_t treeSlices);
@@ -162,7 +165,8 @@ TBAMD_EXPORT int32_t tbmi_forest_tree(intptr_t forest, int32_t tree, float *valu
 TBAMD_EXPORT int32_t tbmi_forest_load_profile(intptr_t forest, const char *profileCSVPath, int64_t *numRows,
                                               double *expectedSteps);
 /* Packs the forest for the given plan and unpacks it again; returns the number of trees that differ
- * from the (comparison-normalised) input, or -1 when the plan cannot hold the model.
+ * from the (comparison-normalised) input, or -1 when the plan cannot hold the model.  groupBytes 0 packs
+ * the global-memory layout (no tree groups) instead.
  * stats[0..4] = groups, bundles, nodes, ldsBytes, paddingTrees. */
 TBAMD_EXPORT int32_t tbmi_pack_roundtrip(intptr_t forest, int32_t rowsPerBlock, int32_t interleave,
                                          int32_t groupBytes, int64_t *stats);

@@ -440,3 +440,81 @@ def test_many_tree_slices_on_small_batches(synth_model, k, rows, slices):
         margins = torch.zeros((rows, 8), dtype=torch.float32, device="cuda")
         runner.run_device_multiclass(dx.data_ptr(), rows, None, margins.data_ptr(), None)
         np.testing.assert_allclose(margins.cpu().numpy(), cpu_oracle.predict(forest, x)[1], rtol=RTOL_SUM, atol=1e-7)
+
+
+# --------------------------------------------------------------------------
+# forests with a tree too big for an LDS tree group: the global-memory walk
+# --------------------------------------------------------------------------
+def big_tree_model(path, num_class, seed=21):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    split = lambda: (rng.integers(0, 12), rng.normal())
+    leaf = lambda: rng.normal(0.0, 0.1)
+    trees = [synth._grow_tree(rng, 14, lambda d, s: 1.0 if d < 13 else 0.6, split, leaf)]        # > 8190 nodes
+    trees += [synth._grow_tree(rng, int(rng.integers(0, 9)), lambda d, s: 0.8, split, leaf, force_root=False)
+              for _ in range(37)]
+    if num_class:
+        info = [int(c) for c in rng.permutation(len(trees)) % num_class]                         # every class has trees
+        synth.write_xgboost_json(path, trees, 12, objective="multi:softmax", num_class=num_class, tree_info=info)
+    else:
+        synth.write_xgboost_json(path, trees, 12, objective="binary:logistic")
+    return path
+
+
+@pytest.mark.parametrize("num_class", [0, 6])
+@pytest.mark.parametrize("rows", [1, 77, 5000])
+def test_trees_too_big_for_lds_walk_from_global_memory(tmp_path, num_class, rows):
+    path = big_tree_model(tmp_path / "big.json", num_class)
+    forest = model_io.load_xgboost_json(path)
+    assert max(len(forest.tree(t)[0]) for t in range(forest.num_trees)) > 8190
+    x = np.random.Generator(np.random.PCG64(rows)).normal(size=(rows, 12)).astype(np.float32)
+    runner = make_runner(path, rows)
+    assert "kernel=global_walk" in runner.describe_plan()
+    check_against_oracle(runner, forest, x)
+    with pytest.raises(RuntimeError, match="does not fit"):
+        runner.set_plan(256, 1, 4, 65536, 1)
+
+
+@pytest.mark.parametrize("plan", [(64, 1, 1), (256, 2, 7), (1024, 8, 3), (128, 4, 1000)])
+@pytest.mark.parametrize("k", [1, 3])
+def test_global_walk_plans_agree(synth_model, k, plan):
+    forest = model_io.load_xgboost_json(synth_model(k))
+    x = synth.CONFIGS[k].batch_rows(1500, seed_offset=6)
+    runner = make_runner(synth_model(k), 1500)
+    runner.set_global_walk_plan(*plan)
+    assert "kernel=global_walk rowsPerBlock=%d" % plan[0] in runner.describe_plan()
+    check_against_oracle(runner, forest, x)
+
+
+@pytest.mark.parametrize("kernel", ["rows_lds", "tree_parallel", "global_walk"])
+def test_classes_without_trees_score_the_initial_value(tmp_path, kernel):
+    """The reference's two sides disagree on a class no tree votes for: its generated code fills every class
+    sum with the initial value before reducing (src/reduction/LowerReduceOps.cpp:1459-1470,
+    src/mlir/LowerToMidLevelIR.cpp:405-428), its scalar check leaves such a class at 0
+    (src/include/DecisionForest.h:526-533).  The kernels follow the generated code."""
+    rng = np.random.Generator(np.random.PCG64(8))
+    split = lambda: (rng.integers(0, 5), rng.normal())
+    trees = [synth._grow_tree(rng, 4, lambda d, s: 0.9, split, lambda: rng.normal(0.0, 0.3)) for _ in range(30)]
+    info = [int(c) for c in rng.choice([0, 2, 3, 5], size=len(trees))]
+    path = tmp_path / "gaps.json"
+    synth.write_xgboost_json(path, trees, 5, objective="multi:softmax", num_class=7, tree_info=info)
+    forest = model_io.load_xgboost_json(path)
+    rows = 600
+    x = rng.normal(size=(rows, 5)).astype(np.float32)
+    runner = make_runner(path, rows)
+    if kernel == "rows_lds":
+        runner.set_plan(64, 2, 2, 4096, 3)
+    elif kernel == "tree_parallel":
+        runner.set_tree_parallel_plan(4, 16, 2, 0, 2)
+    else:
+        runner.set_global_walk_plan(128, 2, 4)
+    assert "kernel=" + kernel in runner.describe_plan()
+    np.testing.assert_array_equal(gpu_leaf_ids(runner, x), cpu_oracle.leaf_ids(forest, x))
+    _, sums = cpu_oracle.predict(forest, x)
+    voted = np.isin(np.arange(7), info)
+    expected = np.where(voted[None, :], sums, forest.initial_value).astype(np.float32)
+    dx = torch.from_numpy(x).cuda()
+    margins = torch.zeros((rows, 7), dtype=torch.float32, device="cuda")
+    classes = torch.zeros((rows,), dtype=torch.int8, device="cuda")
+    runner.run_device_multiclass(dx.data_ptr(), rows, classes.data_ptr(), margins.data_ptr(), None)
+    np.testing.assert_allclose(margins.cpu().numpy(), expected, rtol=RTOL_SUM, atol=1e-7)
+    np.testing.assert_array_equal(classes.cpu().numpy(), cpu_oracle.argmax_generated(expected))

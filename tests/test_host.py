@@ -117,6 +117,16 @@ def test_onnx_comparison_modes_and_encodings(lib, tmp_path, mode, packed):
     lib.tbmi_delete_forest(h)
 
 
+def test_global_layout_round_trips(lib, synth_model):
+    for k in (1, 3, 5):
+        h = load_forest(lib, synth_model(k))
+        stats = (ctypes.c_int64 * 5)()
+        assert lib.tbmi_pack_roundtrip(h, 256, 4, 0, stats) == 0, last_error()
+        forest = model_io.load_xgboost_json(synth_model(k))
+        assert stats[0] == 0 and stats[2] == len(forest.threshold) and stats[3] == 0
+        lib.tbmi_delete_forest(h)
+
+
 def test_pack_rejects_plans_that_cannot_hold_the_model(lib, synth_model):
     h = load_forest(lib, synth_model(5))
     stats = (ctypes.c_int64 * 5)()

@@ -44,6 +44,23 @@ struct alignas(32) DeviceBundle {
   uint32_t reserved;
 };
 
+// Node of the global-memory walk (trees too big for an LDS group): 16 bytes, absolute indices.
+struct DeviceGlobalNode {
+  float value;        // threshold, or the prediction on a leaf
+  uint32_t feature;   // feature index; kGlobalLeaf on a leaf
+  uint32_t left;      // index of the left child in the node array (right = left + 1)
+  int32_t origin;     // node id in the model file's numbering
+};
+constexpr uint32_t kGlobalLeaf = 0xFFFFFFFFu;
+
+// Per-tree record of the global-memory walk.
+struct DeviceGlobalTree {
+  uint32_t root;
+  uint32_t depth;
+  uint32_t classId;
+  int32_t origin;     // tree index in the model file
+};
+
 struct DeviceGroup {
   uint32_t nodeBegin;   // first node of the group in the packed node array
   uint32_t nodeCount;   // multiple of 2 so that the group is a whole number of 16-byte pieces

@@ -29,6 +29,8 @@ struct WalkParams {
   const uint4 *nodes16 = nullptr; // packed nodes viewed as 16-byte pieces
   const DeviceBundle *bundles = nullptr;
   const DeviceGroup *groups = nullptr;
+  const DeviceGlobalNode *globalNodes = nullptr; // global-memory walk only
+  const DeviceGlobalTree *globalTrees = nullptr;
   float *out = nullptr;           // used when the epilogue is fused (1 slice, no classes)
   double *partial = nullptr;      // [partials][rows][max(1, classes)] otherwise
   // leaf-id dump (parity checks only)
@@ -61,6 +63,9 @@ hipError_t LaunchBinRows(const float *x, const float *table, uint8_t *ranks, int
 // Tree-parallel walk: s.rowsPerBlock rows per block (row-major in LDS),
 // s.treeLanes lanes per row; block = rowsPerBlock * treeLanes lanes.
 hipError_t LaunchWalkTreeParallel(const WalkParams &p, int interleave, size_t ldsBytes, hipStream_t stream);
+// Global-memory walk (fallback for trees that do not fit an LDS group): block = s.rowsPerBlock lanes,
+// one per row; p.globalNodes / p.globalTrees instead of groups and bundles.
+hipError_t LaunchWalkGlobal(const WalkParams &p, int interleave, hipStream_t stream);
 hipError_t LaunchFinalize(const FinalizeParams &p, hipStream_t stream);
 
 } // namespace tbamd

@@ -448,6 +448,75 @@ WalkTreeParallelKernel(const float *__restrict__ x, const uint4 *__restrict__ no
 }
 
 // ---------------------------------------------------------------------------
+// Global-memory walk: the fallback for forests with a tree that does not fit one LDS group.  One
+// lane per row; nodes (16 bytes, absolute child indices) and row values are read from global memory
+// through L1/L2, K trees at a time in lock step with an explicit leaf test.  Same accumulation,
+// class flush and tree-slice scheme as the LDS kernels.
+// ---------------------------------------------------------------------------
+template <int K, bool kDump>
+__global__ void __launch_bounds__(1024)
+WalkGlobalKernel(const float *__restrict__ x, const DeviceGlobalNode *__restrict__ nodes,
+                 const DeviceGlobalTree *__restrict__ trees, const WalkScalars s, float *__restrict__ out,
+                 double *__restrict__ partial, int32_t *__restrict__ leafIds) {
+  const int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const bool valid = row < s.rows;
+  const float *xr = x + (valid ? row : s.rows - 1) * s.numFeatures;
+  const int slice = blockIdx.y;
+  const int tBegin = (int)(((int64_t)s.numTrees * slice) / s.treeSlices);
+  const int tEnd = (int)(((int64_t)s.numTrees * (slice + 1)) / s.treeSlices);
+  const int C = s.numClasses;
+  double *partialRow = partial ? partial + ((int64_t)slice * s.rows + (valid ? row : 0)) * (C > 0 ? C : 1) : nullptr;
+  typedef uint32_t Quad __attribute__((ext_vector_type(4)));
+  const Quad *nodeQuads = reinterpret_cast<const Quad *>(nodes);
+
+  double acc = 0.0;
+  int curClass = 0;
+  for (int t0 = tBegin; t0 < tEnd; t0 += K) {
+    uint32_t n[K];
+    uint32_t depth = 0;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const int t = t0 + k < tEnd ? t0 + k : tEnd - 1; // the tail repeats the last tree; its result is dropped
+      n[k] = trees[t].root;
+      depth = trees[t].depth > depth ? trees[t].depth : depth;
+    }
+    for (uint32_t d = 0; d < depth; ++d) {
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        const Quad node = nodeQuads[n[k]];
+        if (node.y != kGlobalLeaf) n[k] = node.z + (xr[node.y] < AsFloat(node.x) ? 0u : 1u);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      if (t0 + k >= tEnd) break;
+      const DeviceGlobalTree tree = trees[t0 + k];
+      const Quad leaf = nodeQuads[n[k]];
+      if (C > 0 && (int)tree.classId != curClass) { // classes arrive in ascending order
+        if (valid) {
+          partialRow[curClass] = acc;
+          for (int c = curClass + 1; c < (int)tree.classId; ++c) partialRow[c] = 0.0;
+        }
+        acc = 0.0;
+        curClass = (int)tree.classId;
+      }
+      acc += (double)AsFloat(leaf.x);
+      if (kDump && valid) leafIds[row * s.numTrees + tree.origin] = (int32_t)leaf.w;
+    }
+  }
+  if (!valid) return;
+  if (C > 0) {
+    partialRow[curClass] = acc;
+    for (int c = curClass + 1; c < C; ++c) partialRow[c] = 0.0;
+  } else if (partial) {
+    partialRow[0] = acc;
+  } else {
+    const double margin = s.initialValue + acc;
+    out[row] = (float)(s.transform == 1 ? 1.0 / (1.0 + exp(-margin)) : margin);
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Rank quantisation of the rows.  For every (row, feature) the kernel counts how many of the
 // feature's sorted distinct split thresholds are <= the value (NaN counts as 255, which no node
 // accepts as "left") and writes the count as one byte into the tile layout the row-parallel kernel
@@ -689,6 +758,33 @@ hipError_t LaunchWalkTreeParallel(const WalkParams &p, int interleave, size_t ld
   case 2: return LaunchTreeParallelK<2>(p, prefetch, grid, block, ldsBytes, stream);
   case 4: return LaunchTreeParallelK<4>(p, prefetch, grid, block, ldsBytes, stream);
   case 8: return LaunchTreeParallelK<8>(p, prefetch, grid, block, ldsBytes, stream);
+  default: return hipErrorInvalidValue;
+  }
+}
+
+namespace {
+template <int K>
+hipError_t LaunchGlobalK(const WalkParams &p, dim3 grid, dim3 block, hipStream_t stream) {
+  if (p.leafIds)
+    WalkGlobalKernel<K, true><<<grid, block, 0, stream>>>(p.x, p.globalNodes, p.globalTrees, p.s, p.out, p.partial, p.leafIds);
+  else
+    WalkGlobalKernel<K, false><<<grid, block, 0, stream>>>(p.x, p.globalNodes, p.globalTrees, p.s, p.out, p.partial, nullptr);
+  return hipGetLastError();
+}
+} // namespace
+
+hipError_t LaunchWalkGlobal(const WalkParams &p, int interleave, hipStream_t stream) {
+  if (p.s.rows <= 0) return hipSuccess;
+  const int threads = p.s.rowsPerBlock;
+  if (threads < 64 || threads > 1024 || threads % 64 != 0) return hipErrorInvalidValue;
+  const int64_t blocks = (p.s.rows + threads - 1) / threads;
+  if (blocks > 0x7FFFFFFF || p.s.treeSlices < 1 || p.s.treeSlices > 65535) return hipErrorInvalidValue;
+  dim3 grid((unsigned)blocks, (unsigned)p.s.treeSlices), block((unsigned)threads);
+  switch (interleave) {
+  case 1: return LaunchGlobalK<1>(p, grid, block, stream);
+  case 2: return LaunchGlobalK<2>(p, grid, block, stream);
+  case 4: return LaunchGlobalK<4>(p, grid, block, stream);
+  case 8: return LaunchGlobalK<8>(p, grid, block, stream);
   default: return hipErrorInvalidValue;
   }
 }

@@ -31,6 +31,7 @@ size_t PackedModel::RowTileBytes() const {
 }
 
 size_t PackedModel::LdsBytes() const {
+  if (plan.kernel == LaunchPlan::Kernel::kGlobalWalk) return 0;
   size_t bytes = RowTileBytes() + (size_t)GroupRegionBytes();
   if (plan.kernel == LaunchPlan::Kernel::kTreeParallel) {
     // cross-wave reduction scratch + per-row, per-class accumulators (doubles)
@@ -91,8 +92,57 @@ LevelOrder MakeLevelOrder(const Tree &tree) {
 
 } // namespace
 
+namespace {
+
+// Global-memory layout: every tree breadth first (siblings adjacent), absolute node indices.
+PackedModel PackForGlobalWalk(const Forest &forest, const LaunchPlan &plan) {
+  if (plan.rowsPerBlock < 64 || plan.rowsPerBlock > 1024 || plan.rowsPerBlock % 64 != 0)
+    throw Error("the global-memory walk needs a block of 64..1024 lanes");
+  PackedModel pm;
+  pm.plan = plan;
+  pm.numFeatures = forest.numFeatures;
+  pm.numClasses = forest.numClasses;
+  pm.numTrees = (int32_t)forest.trees.size();
+  std::vector<int32_t> depth(forest.trees.size());
+  for (size_t t = 0; t < forest.trees.size(); ++t) depth[t] = forest.trees[t].Depth();
+  std::vector<int32_t> order(forest.trees.size());
+  std::iota(order.begin(), order.end(), 0);
+  std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) {
+    const int32_t ca = forest.numClasses > 0 ? forest.trees[a].classId : 0;
+    const int32_t cb = forest.numClasses > 0 ? forest.trees[b].classId : 0;
+    if (ca != cb) return ca < cb;
+    return depth[a] < depth[b];
+  });
+  if (forest.NumNodes() > 0x7FFFFFF0u) throw Error("forest has too many nodes");
+  for (int32_t t : order) {
+    const Tree &tree = forest.trees[t];
+    const LevelOrder lo = MakeLevelOrder(tree);
+    const uint32_t base = (uint32_t)pm.globalNodes.size();
+    pm.globalTrees.push_back(DeviceGlobalTree{base, (uint32_t)depth[t],
+                                              (uint32_t)(forest.numClasses > 0 ? tree.classId : 0), t});
+    for (size_t i = 0; i < lo.order.size(); ++i) {
+      const int32_t n = lo.order[i];
+      DeviceGlobalNode dn;
+      dn.value = tree.value[n];
+      dn.origin = n;
+      if (tree.IsLeaf(n)) {
+        dn.feature = kGlobalLeaf;
+        dn.left = base + (uint32_t)i;
+      } else {
+        dn.feature = (uint32_t)tree.feature[n];
+        dn.left = base + (uint32_t)lo.position[tree.left[n]];
+      }
+      pm.globalNodes.push_back(dn);
+    }
+  }
+  return pm;
+}
+
+} // namespace
+
 PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
   const Forest forest = NormalizeToLessThan(input);
+  if (plan.kernel == LaunchPlan::Kernel::kGlobalWalk) return PackForGlobalWalk(forest, plan);
   const int K = plan.interleave;
   if (K < 1 || K > kMaxInterleave || (K & (K - 1))) throw Error("interleave must be 1, 2, 4 or 8");
   if (plan.kernel == LaunchPlan::Kernel::kRowParallelLds) {
@@ -270,6 +320,35 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
 }
 
 Tree UnpackTree(const PackedModel &pm, int32_t treeIndex) {
+  if (pm.plan.kernel == LaunchPlan::Kernel::kGlobalWalk) {
+    for (const DeviceGlobalTree &gt : pm.globalTrees) {
+      if (gt.origin != treeIndex) continue;
+      Tree tree;
+      tree.classId = (int32_t)gt.classId;
+      std::vector<uint32_t> queue{gt.root};
+      size_t total = 0;
+      for (size_t head = 0; head < queue.size(); ++head) {
+        const DeviceGlobalNode &dn = pm.globalNodes[queue[head]];
+        total = std::max<size_t>(total, (size_t)dn.origin + 1);
+        if (dn.feature != kGlobalLeaf) { queue.push_back(dn.left); queue.push_back(dn.left + 1); }
+      }
+      tree.value.assign(total, 0.f);
+      tree.feature.assign(total, 0);
+      tree.left.assign(total, -1);
+      tree.right.assign(total, -1);
+      for (uint32_t q : queue) {
+        const DeviceGlobalNode &dn = pm.globalNodes[q];
+        tree.value[dn.origin] = dn.value;
+        if (dn.feature != kGlobalLeaf) {
+          tree.feature[dn.origin] = (int32_t)dn.feature;
+          tree.left[dn.origin] = pm.globalNodes[dn.left].origin;
+          tree.right[dn.origin] = pm.globalNodes[dn.left + 1].origin;
+        }
+      }
+      return tree;
+    }
+    throw Error("tree not found in packed model");
+  }
   const int K = pm.plan.interleave;
   const uint32_t featureStride = pm.plan.FeatureStride();
   for (const DeviceGroup &g : pm.groups)

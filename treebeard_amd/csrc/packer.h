@@ -12,13 +12,15 @@ namespace tbamd {
 //
 //  kRowParallelLds: one lane per row, rowsPerBlock lanes per block, the block's
 //    rows transposed in LDS, every lane walks all trees (K at a time).
+//  kGlobalWalk:     one lane per row, rows and nodes read from global memory (through L1/L2); the
+//    fallback for forests with a tree that does not fit one 64 KB LDS group.
 //  kTreeParallel:   rowsPerBlock rows per block kept row-major in LDS and
 //    treeLanes lanes per row that split the trees between them; per-row sums are
 //    reduced across lanes (wave shuffles, then LDS across waves).  For models
 //    whose rows are too wide to transpose into LDS and for batches too small to
 //    fill the chip with one lane per row.
 struct LaunchPlan {
-  enum class Kernel : int32_t { kRowParallelLds = 0, kTreeParallel = 1 };
+  enum class Kernel : int32_t { kRowParallelLds = 0, kTreeParallel = 1, kGlobalWalk = 2 };
   Kernel kernel = Kernel::kRowParallelLds;
   int32_t rowsPerBlock = 256;   // row-parallel: rows (= lanes per tree thread) per block, power of two
   int32_t treeThreads = 1;      // row-parallel: lanes in different waves that share a row; block = rowsPerBlock * treeThreads
@@ -33,6 +35,7 @@ struct LaunchPlan {
   bool quantizedRows = false;
 
   int32_t ThreadsPerBlock() const {
+    if (kernel == Kernel::kGlobalWalk) return rowsPerBlock;
     return kernel == Kernel::kTreeParallel ? rowsPerBlock * treeLanes : rowsPerBlock * treeThreads;
   }
   // Distance in LDS between feature f and f+1 of one row, in the units node offsets use.
@@ -55,6 +58,9 @@ struct PackedModel {
   std::vector<int32_t> nodeOrigin; // per packed node: original node id inside its tree (-1: null leaf)
   std::vector<int32_t> slotTree;   // per bundle slot: original tree index, -1 for a padding tree
   uint32_t maxGroupNodes = 0;
+  // kGlobalWalk only:
+  std::vector<DeviceGlobalNode> globalNodes;
+  std::vector<DeviceGlobalTree> globalTrees; // ordered by (class, depth)
   // Rank quantisation (plan.quantizedRows): per feature the sorted distinct thresholds, stored for the
   // binning kernel as [featureChunk][k][binChunkFeatures] with NaN behind a feature's last threshold;
   // binTableDepth = 2^n - 1 entries per feature.

@@ -81,7 +81,11 @@ void InferenceRunner::FreeModel() {
   (void)hipFree(m_dNodeOrigin);
   (void)hipFree(m_dSlotTree);
   (void)hipFree(m_dBinTable);
+  (void)hipFree(m_dGlobalNodes);
+  (void)hipFree(m_dGlobalTrees);
   m_dBinTable = nullptr;
+  m_dGlobalNodes = nullptr;
+  m_dGlobalTrees = nullptr;
   m_dNodes = nullptr;
   m_dBundles = nullptr;
   m_dGroups = nullptr;
@@ -90,6 +94,12 @@ void InferenceRunner::FreeModel() {
 }
 
 void InferenceRunner::UploadModel() {
+  if (m_model.plan.kernel == LaunchPlan::Kernel::kGlobalWalk) {
+    m_model.plan.treeSlices = std::max(1, std::min<int32_t>(m_model.plan.treeSlices, (int32_t)m_model.globalTrees.size()));
+    m_dGlobalNodes = Upload(m_model.globalNodes, "upload nodes");
+    m_dGlobalTrees = Upload(m_model.globalTrees, "upload trees");
+    return;
+  }
   // treeSlices never exceeds the number of groups the packer produced
   m_model.plan.treeSlices = std::max(1, std::min<int32_t>(m_model.plan.treeSlices, (int32_t)m_model.groups.size()));
   if (m_model.LdsBytes() > (size_t)m_limits.ldsBytesPerBlock) throw Error("launch plan exceeds the LDS of one workgroup");
@@ -151,6 +161,7 @@ void InferenceRunner::EnsureStaging() {
 
 hipError_t InferenceRunner::LaunchWalk(const WalkParams &p) const {
   const LaunchPlan &plan = m_model.plan;
+  if (plan.kernel == LaunchPlan::Kernel::kGlobalWalk) return LaunchWalkGlobal(p, plan.interleave, m_stream);
   if (plan.kernel == LaunchPlan::Kernel::kTreeParallel)
     return LaunchWalkTreeParallel(p, plan.interleave, m_model.LdsBytes(), m_stream);
   const int tileMode = plan.quantizedRows ? 2 : (plan.featureOffsetInWords ? 1 : 0);
@@ -172,6 +183,8 @@ WalkParams InferenceRunner::MakeWalkParams(const float *deviceInputs, int64_t ro
   p.s.treeLanes = m_model.plan.treeLanes;
   p.s.initialValue = m_forest.initialValue;
   p.x = deviceInputs;
+  p.globalNodes = m_dGlobalNodes;
+  p.globalTrees = m_dGlobalTrees;
   p.nodes16 = reinterpret_cast<const uint4 *>(m_dNodes);
   p.bundles = m_dBundles;
   p.groups = m_dGroups;
@@ -371,7 +384,10 @@ double InferenceRunner::AutoTune(const float *deviceInputs, int64_t rows) {
 std::string InferenceRunner::DescribePlan() const {
   std::ostringstream os;
   const LaunchPlan &p = m_model.plan;
-  os << "kernel=" << (p.kernel == LaunchPlan::Kernel::kTreeParallel ? "tree_parallel" : "rows_lds")
+  os << "kernel="
+     << (p.kernel == LaunchPlan::Kernel::kTreeParallel ? "tree_parallel"
+         : p.kernel == LaunchPlan::Kernel::kGlobalWalk ? "global_walk"
+                                                       : "rows_lds")
      << " rowsPerBlock=" << p.rowsPerBlock << " treeThreads=" << p.treeThreads << " treeLanes=" << p.treeLanes
      << " interleave=" << p.interleave
      << " groupBytes=" << p.groupBytes << " treeSlices=" << p.treeSlices

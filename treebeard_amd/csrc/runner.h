@@ -87,6 +87,8 @@ private:
   hipEvent_t m_pieceReady[8] = {};
   hipEvent_t m_evStart = nullptr, m_evStop = nullptr;
 
+  DeviceGlobalNode *m_dGlobalNodes = nullptr;
+  DeviceGlobalTree *m_dGlobalTrees = nullptr;
   DeviceNode *m_dNodes = nullptr;
   DeviceBundle *m_dBundles = nullptr;
   DeviceGroup *m_dGroups = nullptr;

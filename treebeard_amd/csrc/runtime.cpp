@@ -380,6 +380,22 @@ int32_t tbmi_set_tree_parallel_plan(intptr_t h, int32_t rowsPerBlock, int32_t tr
       -1);
 }
 
+int32_t tbmi_set_global_walk_plan(intptr_t h, int32_t rowsPerBlock, int32_t interleave, int32_t treeSlices) {
+  return Guard(
+      [&] {
+        InferenceRunner *r = Runner(h);
+        LaunchPlan plan;
+        plan.kernel = LaunchPlan::Kernel::kGlobalWalk;
+        plan.rowsPerBlock = rowsPerBlock > 0 ? rowsPerBlock : 256;
+        plan.interleave = interleave > 0 ? interleave : 4;
+        plan.treeSlices = treeSlices > 0 ? treeSlices : 1;
+        plan.groupBytes = 0;
+        r->Repack(plan);
+        return 0;
+      },
+      -1);
+}
+
 int32_t tbmi_set_quantized_plan(intptr_t h, int32_t treeThreads, int32_t interleave, int32_t groupBytes,
                                 int32_t treeSlices) {
   return Guard(
@@ -518,6 +534,7 @@ int32_t tbmi_pack_roundtrip(intptr_t h, int32_t rowsPerBlock, int32_t interleave
         plan.interleave = interleave;
         plan.groupBytes = groupBytes;
         plan.featureOffsetInWords = (int64_t)(f->numFeatures + 1) * rowsPerBlock * 4 > 0xFFFF;
+        if (groupBytes == 0) plan.kernel = LaunchPlan::Kernel::kGlobalWalk; // the layout without tree groups
         PackedModel pm = PackForest(*f, plan);
         const Forest norm = NormalizeToLessThan(*f);
         int32_t mismatches = 0;
@@ -535,7 +552,7 @@ int32_t tbmi_pack_roundtrip(intptr_t h, int32_t rowsPerBlock, int32_t interleave
           for (int32_t s : pm.slotTree) padding += s < 0;
           stats[0] = (int64_t)pm.groups.size();
           stats[1] = (int64_t)pm.bundles.size();
-          stats[2] = (int64_t)pm.nodes.size();
+          stats[2] = (int64_t)(pm.nodes.size() + pm.globalNodes.size());
           stats[3] = (int64_t)pm.LdsBytes();
           stats[4] = padding;
         }

@@ -78,6 +78,21 @@ LaunchPlan ChooseTreeParallelPlan(const Forest &forest, int64_t batchSize, const
 
 LaunchPlan ChoosePlan(const Forest &forest, int64_t batchSize, const GPUAutoScheduleOptions *ov,
                       const DeviceLimits &limits) {
+  if ((BiggestTreeNodes(forest) + 2) * kNodeBytes > 65536) {
+    // A tree that cannot sit in one LDS group: walk from global memory.
+    LaunchPlan plan;
+    plan.kernel = LaunchPlan::Kernel::kGlobalWalk;
+    plan.rowsPerBlock = 256;
+    plan.interleave = 4;
+    if (ov && ov->treeWalkInterleaveFactor > 0)
+      plan.interleave = std::min(kMaxInterleave, FloorPow2(ov->treeWalkInterleaveFactor));
+    const int64_t rowBlocks = std::max<int64_t>(1, (batchSize + 255) / 256);
+    int64_t slices = 1;
+    if (rowBlocks < 4LL * limits.computeUnits) slices = (4LL * limits.computeUnits + rowBlocks - 1) / rowBlocks;
+    plan.treeSlices = (int32_t)std::max<int64_t>(1, std::min<int64_t>(slices, (int64_t)forest.trees.size()));
+    plan.groupBytes = 0;
+    return plan;
+  }
   bool fitsTransposed = false;
   {
     bool words = false;
@@ -172,6 +187,14 @@ std::vector<LaunchPlan> CandidatePlans(const Forest &forest, int64_t batchSize, 
   std::vector<LaunchPlan> out;
   LaunchPlan base = ChoosePlan(forest, batchSize, nullptr, limits);
   out.push_back(base);
+  if (base.kernel == LaunchPlan::Kernel::kGlobalWalk) {
+    for (int32_t k : {1, 2, 8}) {
+      LaunchPlan p = base;
+      p.interleave = k;
+      out.push_back(p);
+    }
+    return out;
+  }
   if (base.kernel == LaunchPlan::Kernel::kTreeParallel) {
     for (int32_t lanes : {base.treeLanes / 2, base.treeLanes * 2})
       for (int32_t k : {1, 2}) {

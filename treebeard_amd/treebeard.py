@@ -306,6 +306,10 @@ class TreebeardInferenceRunner:
                  "tbmi_time_kernels")
         return walk.value, fin.value, pre.value
 
+    def set_global_walk_plan(self, rows_per_block=256, interleave=4, tree_slices=1):
+        self._rc(_lib().tbmi_set_global_walk_plan(self.inferenceRunner, rows_per_block, interleave, tree_slices),
+                 "tbmi_set_global_walk_plan")
+
     def set_quantized_plan(self, tree_threads=8, interleave=4, group_bytes=0, tree_slices=1):
         self._rc(_lib().tbmi_set_quantized_plan(self.inferenceRunner, tree_threads, interleave, group_bytes,
                                                 tree_slices), "tbmi_set_quantized_plan")
