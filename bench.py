@@ -37,7 +37,7 @@ def main():
                     help="also run one plain device copy of this many MiB (counter calibration for rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this engine runs on ONE GPU (rows shard trivially; see DESIGN.md) - use --gpus 1")
+        sys.exit("bench.py: this engine runs on ONE GPU (a batch would shard by rows, each GPU holding the whole model) - use --gpus 1")
 
     import numpy as np
     import torch
