@@ -96,6 +96,21 @@ def main():
     hbm_ms = walk_ms + bin_ms if quantized else walk_ms
     hbm_gbs = hbm_bytes_row * rows / (hbm_ms * 1e-3) / 1e9
     lds_gbs = lds_bytes_row * rows / (walk_ms * 1e-3) / 1e9
+    # measured alongside the published peak: a plain device copy (bytes read + bytes written per second)
+    # (left out of counter-calibration runs, which want exactly one copy of known size in their trace)
+    copy_gbs = None
+    if not args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for _ in range(5):
+            dst.copy_(src)
+        ev1.record()
+        torch.cuda.synchronize()
+        copy_gbs = 5 * 2 * (1 << 30) / (ev0.elapsed_time(ev1) * 1e-3) / 1e9
+        del src, dst
     traffic = None
     traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(traffic_file):
@@ -113,7 +128,9 @@ def main():
                      "frac": hbm_gbs / HBM_PEAK_GBS, "traffic": traffic,
                      "kernel": ("BinRowsKernel+" if quantized else "") + kernel,
                      "kernel_ms": walk_ms, "finalize_ms": fin_ms, "bin_ms": bin_ms,
-                     "algorithmic_bytes_per_row": hbm_bytes_row},
+                     "algorithmic_bytes_per_row": hbm_bytes_row,
+                     "measured_copy_gbs": copy_gbs,
+                     "frac_of_measured_copy": hbm_gbs / copy_gbs if copy_gbs else None},
         "roofline_binding": {"bound": binding, "achieved": lds_gbs if binding == "lds" else hbm_gbs,
                              "peak": LDS_PEAK_GBS if binding == "lds" else HBM_PEAK_GBS, "unit": "GB/s",
                              "frac": (lds_gbs / LDS_PEAK_GBS) if binding == "lds" else (hbm_gbs / HBM_PEAK_GBS),
@@ -150,6 +167,11 @@ def main():
         cpu_s = time.perf_counter() - t0
         line["cpu_baseline"] = {"value": cpu_rows / cpu_s, "unit": "rows/s", "cores": threads, "kind": "port",
                                 "sample": "first %d rows of the same batch; %s" % (cpu_rows, what)}
+        # the scalar walker (one thread, one row at a time, every tree) on a small sample, for scale
+        scalar_rows = int(min(cpu_rows, 2048))
+        t0 = time.perf_counter()
+        cpu_oracle.predict(forest, x[:scalar_rows], threads=1)
+        line["cpu_baseline"]["scalar_one_thread_rows_per_s"] = scalar_rows / (time.perf_counter() - t0)
         got = out[:cpu_rows].cpu().numpy().astype(np.float32)
         line["cpu_baseline"]["max_abs_diff_vs_gpu"] = float(np.abs(got - cpu_out).max())
     print(json.dumps(line))

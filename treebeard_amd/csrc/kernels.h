@@ -57,7 +57,7 @@ struct FinalizeParams {
 // 4 bytes, 2 one-byte rank tile (p.x then points at the output of LaunchBinRows; 64 rows per block).
 hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, int tileMode, size_t ldsBytes, hipStream_t stream);
 // Rank-quantises rows x[rows][numFeatures] into ranks[ceil(rows/64)][numFeatures][64] (bytes) with the
-// packer's threshold table ([chunk][k][chunkFeatures], NaN padded, tableDepth = 2^n - 1).
+// packer's threshold table ([chunk][k][64], +inf padded, tableDepth = 2^n - 1).
 hipError_t LaunchBinRows(const float *x, const float *table, uint8_t *ranks, int64_t rows, int numFeatures,
                          int tableDepth, int chunkFeatures, hipStream_t stream);
 // Tree-parallel walk: s.rowsPerBlock rows per block (row-major in LDS),

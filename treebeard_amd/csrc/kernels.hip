@@ -184,9 +184,9 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
   // Register double buffer for the next tree group.  Loads are unconditional
   // (index clamped) so that they stay in flight across the walk.
   U32x4 fetched[PF];
-#define TBAMD_PREFETCH_GROUP(G)                                                                                        \
+#define TBAMD_PREFETCH_GROUP(NEXTGRP)                                                                                  \
   {                                                                                                                    \
-    const DeviceGroup nextGrp = groups[(G)];                                                                           \
+    const DeviceGroup nextGrp = (NEXTGRP);                                                                             \
     const U32x4 *src = reinterpret_cast<const U32x4 *>(nodes16) + (nextGrp.nodeBegin >> 1);                            \
     const int last = (int)(nextGrp.nodeCount >> 1) - 1;                                                                \
     _Pragma("unroll") for (int i = 0; i < PF; ++i) {                                                                   \
@@ -213,7 +213,7 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
     }                                                                                                                  \
     acc = 0.0;                                                                                                         \
   }
-  if (gBegin < gEnd) TBAMD_PREFETCH_GROUP(gBegin)
+  if (gBegin < gEnd) TBAMD_PREFETCH_GROUP(groups[gBegin])
 
   for (int g = gBegin; g < gEnd; ++g) {
     const DeviceGroup grp = groups[g];
@@ -228,7 +228,7 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
       }
     }
     __syncthreads();
-    if (g + 1 < gEnd) TBAMD_PREFETCH_GROUP(g + 1) // in flight while this group is walked
+    if (g + 1 < gEnd) TBAMD_PREFETCH_GROUP(groups[g + 1]) // in flight while this group is walked
 
     // Bundles are sorted by class; a segment is a run of bundles of one class.
     uint32_t b0 = 0;
@@ -357,9 +357,9 @@ WalkTreeParallelKernel(const float *__restrict__ x, const uint4 *__restrict__ no
 
   // Register double buffer for the next tree group (loads stay in flight across the walk).
   U32x4 fetched[PF];
-#define TBAMD_PREFETCH_GROUP(G)                                                                                        \
+#define TBAMD_PREFETCH_GROUP(NEXTGRP)                                                                                  \
   {                                                                                                                    \
-    const DeviceGroup nextGrp = groups[(G)];                                                                           \
+    const DeviceGroup nextGrp = (NEXTGRP);                                                                             \
     const U32x4 *src = reinterpret_cast<const U32x4 *>(nodes16) + (nextGrp.nodeBegin >> 1);                            \
     const int last = (int)(nextGrp.nodeCount >> 1) - 1;                                                                \
     _Pragma("unroll") for (int i = 0; i < PF; ++i) {                                                                   \
@@ -367,7 +367,7 @@ WalkTreeParallelKernel(const float *__restrict__ x, const uint4 *__restrict__ no
       fetched[i] = src[idx < last ? idx : last];                                                                       \
     }                                                                                                                  \
   }
-  if (gBegin < gEnd) TBAMD_PREFETCH_GROUP(gBegin)
+  if (gBegin < gEnd) TBAMD_PREFETCH_GROUP(groups[gBegin])
 
   for (int g = gBegin; g < gEnd; ++g) {
     const DeviceGroup grp = groups[g];
@@ -382,7 +382,7 @@ WalkTreeParallelKernel(const float *__restrict__ x, const uint4 *__restrict__ no
       }
     }
     __syncthreads();
-    if (g + 1 < gEnd) TBAMD_PREFETCH_GROUP(g + 1)
+    if (g + 1 < gEnd) TBAMD_PREFETCH_GROUP(groups[g + 1])
 
     // bundles are sorted by class: handle one class segment at a time
     uint32_t b0 = 0;
@@ -518,72 +518,125 @@ WalkGlobalKernel(const float *__restrict__ x, const DeviceGlobalNode *__restrict
 
 // ---------------------------------------------------------------------------
 // Rank quantisation of the rows.  For every (row, feature) the kernel counts how many of the
-// feature's sorted distinct split thresholds are <= the value (NaN counts as 255, which no node
-// accepts as "left") and writes the count as one byte into the tile layout the row-parallel kernel
-// copies verbatim: [block of 64 rows][feature][row].  The block owns a chunk of features, whose
-// threshold table sits in LDS as [k][feature], and walks the row blocks.  Four consecutive lanes
-// share a feature and take 16 rows of the row block each, so a lane produces exactly one 16-byte
-// piece of the tile and a wave's store covers 1 KB of contiguous tile (16 features x 64 rows).
+// feature's sorted distinct split thresholds are <= the value and writes the count as one byte into
+// the tile layout the row-parallel kernel copies verbatim: [block of 64 rows][feature][row].  The
+// table is padded with +inf up to 2^n - 1 entries; NaN and +inf count all of them (the largest rank,
+// above every node's threshold index, so they go right at every node like the f32 compare sends
+// them).  Rows past the end of the batch in the last block get the ranks of the last row; the walk
+// never stores their results.
+//
+// A block owns a chunk of 64 features, whose threshold table sits in LDS as [k][feature]; its waves
+// take 64-row blocks in turn.  A lane owns ONE feature of the chunk: whatever level of the search a
+// lane is at, lane i reads bank i, so the table reads never conflict, and a wave's row load is 256
+// contiguous bytes.  The lane's 64 result bytes pass through a per-wave LDS area (80-byte lane
+// stride: conflict-free 16-byte writes) so that the wave stores its 4 KB of tile in four contiguous
+// 1 KB pieces.
 // ---------------------------------------------------------------------------
-constexpr int kBinRows = 64;       // rows per tile = rows per block of the quantised walk
-constexpr int kBinRowsPerLane = 16;
+constexpr int kBinRows = 64;        // rows per tile = rows per block of the quantised walk
+constexpr int kBinFeatures = 64;    // features per block = lanes per wave
+constexpr int kBinRowsPerPass = 16; // rows a lane searches side by side
+constexpr int kBinWaves = 8;
+constexpr int kBinLaneStride = 80;  // bytes of staging per lane (64 used)
 
-__global__ void __launch_bounds__(1024)
-BinRowsKernel(const float *__restrict__ x, const float *__restrict__ table, uint8_t *__restrict__ ranks,
-              int64_t rows, int F, int depth, int rowBlocksPerBlock) {
-  extern __shared__ __align__(16) unsigned char lds[];
-  float *tab = reinterpret_cast<float *>(lds);
-  const int tid = threadIdx.x;
-  const int FC = blockDim.x >> 2; // features per block
-  const int fl = tid >> 2;        // feature inside the chunk
-  const int sub = tid & 3;        // which 16 rows of the row block
-  const int f = blockIdx.x * FC + fl;
-  {
-    const float *src = table + (int64_t)blockIdx.x * depth * FC;
-    for (int i = tid; i < depth * FC; i += blockDim.x) tab[i] = src[i];
+// Sixteen rows of one feature, all loads in flight; rows past the batch re-read the last row.
+__device__ __forceinline__ void BinLoadRows(const float *__restrict__ x, int64_t rows, int F, int feature, int64_t rowBase,
+                                            float (&v)[kBinRowsPerPass]) {
+#pragma unroll
+  for (int u = 0; u < kBinRowsPerPass; ++u) {
+    const int64_t row = rowBase + u;
+    v[u] = x[(row < rows ? row : rows - 1) * F + feature];
   }
-  __syncthreads();
+}
+
+// Ranks of sixteen values of the lane's feature, left as one 16-byte piece at LDS address `piece`.
+// Branch-free binary search on byte offsets into the [k][feature] table (lane offset included); every
+// level first issues the reads of all rows, then consumes them, so a wave keeps 16 LDS reads in flight.
+template <int kLevels>
+__device__ __forceinline__ void BinSearchRows(const float (&v)[kBinRowsPerPass], uint32_t laneBytes, unsigned char *piece) {
+  typedef uint32_t Piece __attribute__((ext_vector_type(4)));
+  constexpr uint32_t strideBytes = kBinFeatures * 4u; // one table level
+  uint32_t pos[kBinRowsPerPass];
+#pragma unroll
+  for (int u = 0; u < kBinRowsPerPass; ++u) pos[u] = laneBytes;
+#pragma unroll
+  for (int level = kLevels - 1; level >= 0; --level) {
+    const uint32_t step = strideBytes << level;
+    float probe[kBinRowsPerPass];
+#pragma unroll
+    for (int u = 0; u < kBinRowsPerPass; ++u) probe[u] = LdsLoadFloat(pos[u] + (step - strideBytes));
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < kBinRowsPerPass; ++u) pos[u] += !(v[u] < probe[u]) ? step : 0u; // NaN: every step taken
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // byte 1 of every offset is the rank (offset = rank * 256 + lane * 4): gather four of them per word
+  uint32_t packed[kBinRowsPerPass / 4];
+#pragma unroll
+  for (int i = 0; i < kBinRowsPerPass / 4; ++i) {
+    const uint32_t lo = __builtin_amdgcn_perm(pos[4 * i + 1], pos[4 * i], 0x0c0c0501u);
+    const uint32_t hi = __builtin_amdgcn_perm(pos[4 * i + 3], pos[4 * i + 2], 0x0c0c0501u);
+    packed[i] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+  }
+  *reinterpret_cast<Piece *>(piece) = Piece{packed[0], packed[1], packed[2], packed[3]};
+}
+
+template <int kLevels> // search depth: the table holds 2^kLevels - 1 thresholds per feature
+__global__ void __launch_bounds__(kBinWaves * 64)
+BinRowsKernel(const float *__restrict__ x, const float *__restrict__ table, uint8_t *__restrict__ ranks,
+              int64_t rows, int F, int rowBlocksPerBlock) {
+  extern __shared__ __align__(16) unsigned char lds[];
+  typedef uint32_t Piece __attribute__((ext_vector_type(4)));
+  static_assert(kBinRows == 4 * kBinRowsPerPass, "four passes per row block");
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int f0 = blockIdx.x * kBinFeatures;
+  const int f = f0 + lane;
+  constexpr int depth = (1 << kLevels) - 1;
+  constexpr uint32_t tableBytes = (uint32_t)depth * kBinFeatures * 4u;
+  {
+    float *tab = reinterpret_cast<float *>(lds);
+    const float *src = table + (int64_t)blockIdx.x * depth * kBinFeatures;
+    for (int i = tid; i < depth * kBinFeatures; i += kBinWaves * 64) tab[i] = src[i];
+  }
+  __syncthreads(); // the only block-wide barrier: from here on the waves run on their own
+  unsigned char *stage = lds + tableBytes + (uint32_t)wave * (64u * kBinLaneStride);
+  unsigned char *mine = stage + lane * kBinLaneStride;
   const int64_t numRowBlocks = (rows + kBinRows - 1) / kBinRows;
   const int64_t rbBegin = (int64_t)blockIdx.y * rowBlocksPerBlock;
   const int64_t rbEnd = rbBegin + rowBlocksPerBlock < numRowBlocks ? rbBegin + rowBlocksPerBlock : numRowBlocks;
   const int fClamped = f < F ? f : F - 1;
-  const uint32_t strideBytes = (uint32_t)FC * 4u;                  // one table level
-  const uint32_t laneBytes = (uint32_t)fl * 4u;
-  const uint32_t halfBytes = (uint32_t)((depth + 1) >> 1) * strideBytes; // depth = 2^n - 1
-  int shift = 0;
-  while ((1u << shift) < strideBytes) ++shift;                     // FC is a power of two
-  for (int64_t rb = rbBegin; rb < rbEnd; ++rb) {
-    const int64_t rowBase = rb * kBinRows + sub * kBinRowsPerLane;
-    float v[kBinRowsPerLane];
+  const uint32_t laneBytes = (uint32_t)lane * 4u;
+  // The rows of the next pass are requested before the current pass is searched (two register
+  // buffers), so that the wave always has loads in flight.
+  float va[kBinRowsPerPass], vb[kBinRowsPerPass];
+  int64_t rb = rbBegin + wave;
+  if (rb < rbEnd) BinLoadRows(x, rows, F, fClamped, rb * kBinRows, va);
+  for (; rb < rbEnd; rb += kBinWaves) {
+    const int64_t rowBase = rb * kBinRows;
+    BinLoadRows(x, rows, F, fClamped, rowBase + kBinRowsPerPass, vb);
+    BinSearchRows<kLevels>(va, laneBytes, mine);
+    BinLoadRows(x, rows, F, fClamped, rowBase + 2 * kBinRowsPerPass, va);
+    BinSearchRows<kLevels>(vb, laneBytes, mine + 16);
+    BinLoadRows(x, rows, F, fClamped, rowBase + 3 * kBinRowsPerPass, vb);
+    BinSearchRows<kLevels>(va, laneBytes, mine + 32);
+    const int64_t rbNext = rb + kBinWaves < rbEnd ? rb + kBinWaves : rb; // (the last block re-reads its own rows)
+    BinLoadRows(x, rows, F, fClamped, rbNext * kBinRows, va);
+    BinSearchRows<kLevels>(vb, laneBytes, mine + 48);
+    // the wave's 64 features x 64 rows leave as contiguous 16-byte pieces (piece = feature * 4 + pass)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    uint8_t *dst = ranks + (rb * F + f0) * kBinRows;
 #pragma unroll
-    for (int u = 0; u < kBinRowsPerLane; ++u) { // all loads in flight; rows past the batch re-read the last row
-      const int64_t row = rowBase + u;
-      v[u] = x[(row < rows ? row : rows - 1) * F + fClamped];
+    for (int j = 0; j < 4; ++j) {
+      const int piece = j * 64 + lane;
+      const Piece value = *reinterpret_cast<const Piece *>(stage + (piece >> 2) * kBinLaneStride + (piece & 3) * 16);
+      if (f0 + (piece >> 2) < F) *reinterpret_cast<Piece *>(dst + piece * 16) = value;
     }
-    // branch-free binary search on byte offsets, the 16 rows side by side so that their LDS reads overlap
-    uint32_t pos[kBinRowsPerLane];
-#pragma unroll
-    for (int u = 0; u < kBinRowsPerLane; ++u) pos[u] = 0;
-    for (uint32_t step = halfBytes; step >= strideBytes; step >>= 1) {
-      const uint32_t probe = step - strideBytes + laneBytes;
-#pragma unroll
-      for (int u = 0; u < kBinRowsPerLane; ++u) pos[u] += LdsLoadFloat(pos[u] + probe) <= v[u] ? step : 0u;
-    }
-    uint32_t packed[kBinRowsPerLane / 4];
-#pragma unroll
-    for (int i = 0; i < kBinRowsPerLane / 4; ++i) packed[i] = 0;
-#pragma unroll
-    for (int u = 0; u < kBinRowsPerLane; ++u) {
-      uint32_t rank = pos[u] >> shift;
-      if (v[u] != v[u]) rank = 255u;
-      if (rowBase + u >= rows) rank = 0u;
-      packed[u >> 2] |= rank << (8 * (u & 3));
-    }
-    if (f < F) {
-      typedef uint32_t Piece __attribute__((ext_vector_type(4)));
-      *reinterpret_cast<Piece *>(ranks + (rb * F + f) * kBinRows + sub * kBinRowsPerLane) =
-          Piece{packed[0], packed[1], packed[2], packed[3]};
-    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier(); // the staging area is rewritten by the next row block
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
 }
 
@@ -792,23 +845,38 @@ hipError_t LaunchWalkGlobal(const WalkParams &p, int interleave, hipStream_t str
 hipError_t LaunchBinRows(const float *x, const float *table, uint8_t *ranks, int64_t rows, int numFeatures,
                          int tableDepth, int chunkFeatures, hipStream_t stream) {
   if (rows <= 0) return hipSuccess;
-  if (chunkFeatures != 64 && chunkFeatures != 128 && chunkFeatures != 256) return hipErrorInvalidValue;
-  const size_t ldsBytes = (size_t)tableDepth * chunkFeatures * sizeof(float);
+  if (chunkFeatures != kBinFeatures) return hipErrorInvalidValue;
+  const size_t ldsBytes = (size_t)tableDepth * kBinFeatures * sizeof(float) + (size_t)kBinWaves * 64 * kBinLaneStride;
   if (ldsBytes > 160 * 1024) return hipErrorInvalidValue;
   const int64_t rowBlocks = (rows + kBinRows - 1) / kBinRows;
-  const int chunks = (numFeatures + chunkFeatures - 1) / chunkFeatures;
-  // enough blocks to fill the chip, each amortising its table load over several row blocks
+  const int chunks = (numFeatures + kBinFeatures - 1) / kBinFeatures;
+  // enough blocks to fill the chip, each amortising its table load over several row blocks per wave
   int64_t perBlock = (rowBlocks * chunks + 2047) / 2048;
-  if (perBlock < 1) perBlock = 1;
-  if (perBlock > 64) perBlock = 64;
+  if (perBlock < kBinWaves) perBlock = kBinWaves;
+  if (perBlock > 64 * kBinWaves) perBlock = 64 * kBinWaves;
   const int64_t gridY = (rowBlocks + perBlock - 1) / perBlock;
   if (gridY > 65535) return hipErrorInvalidValue;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&BinRowsKernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
-  if (e != hipSuccess) return e;
-  BinRowsKernel<<<dim3((unsigned)chunks, (unsigned)gridY), dim3((unsigned)chunkFeatures * 4u), ldsBytes, stream>>>(
-      x, table, ranks, rows, numFeatures, tableDepth, (int)perBlock);
-  return hipGetLastError();
+  const dim3 grid((unsigned)chunks, (unsigned)gridY), block(kBinWaves * 64);
+#define TBAMD_BIN_CASE(LEVELS)                                                                                         \
+  case (1 << LEVELS) - 1: {                                                                                            \
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&BinRowsKernel<LEVELS>),                         \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);                    \
+    if (e != hipSuccess) return e;                                                                                     \
+    BinRowsKernel<LEVELS><<<grid, block, ldsBytes, stream>>>(x, table, ranks, rows, numFeatures, (int)perBlock);       \
+    return hipGetLastError();                                                                                          \
+  }
+  switch (tableDepth) {
+    TBAMD_BIN_CASE(1)
+    TBAMD_BIN_CASE(2)
+    TBAMD_BIN_CASE(3)
+    TBAMD_BIN_CASE(4)
+    TBAMD_BIN_CASE(5)
+    TBAMD_BIN_CASE(6)
+    TBAMD_BIN_CASE(7)
+    TBAMD_BIN_CASE(8)
+  default: return hipErrorInvalidValue;
+  }
+#undef TBAMD_BIN_CASE
 }
 
 hipError_t LaunchFinalize(const FinalizeParams &p, hipStream_t stream) {

@@ -185,13 +185,11 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
     int32_t depth = 1;
     while ((size_t)depth < most) depth = depth * 2 + 1; // 2^n - 1 >= most
     pm.binTableDepth = depth;
-    // features per block of the binning kernel: two blocks per CU when the table allows it
-    int32_t chunk = 256;
-    while (chunk > 64 && (int64_t)chunk * depth * 4 > 72 * 1024) chunk /= 2;
-    if ((int64_t)chunk * depth * 4 > 144 * 1024) throw Error("threshold table does not fit LDS");
+    // features per block of the binning kernel: one per lane of a wave
+    const int32_t chunk = 64;
     pm.binChunkFeatures = chunk;
     const int32_t chunks = (forest.numFeatures + chunk - 1) / chunk;
-    pm.binThresholds.assign((size_t)chunks * depth * chunk, std::numeric_limits<float>::quiet_NaN());
+    pm.binThresholds.assign((size_t)chunks * depth * chunk, std::numeric_limits<float>::infinity());
     for (int32_t f = 0; f < forest.numFeatures; ++f)
       for (size_t k = 0; k < ranks[f].size(); ++k)
         pm.binThresholds[((size_t)(f / chunk) * depth + k) * chunk + (f % chunk)] = ranks[f][k];

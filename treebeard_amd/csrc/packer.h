@@ -62,7 +62,7 @@ struct PackedModel {
   std::vector<DeviceGlobalNode> globalNodes;
   std::vector<DeviceGlobalTree> globalTrees; // ordered by (class, depth)
   // Rank quantisation (plan.quantizedRows): per feature the sorted distinct thresholds, stored for the
-  // binning kernel as [featureChunk][k][binChunkFeatures] with NaN behind a feature's last threshold;
+  // binning kernel as [featureChunk][k][binChunkFeatures] with +inf behind a feature's last threshold;
   // binTableDepth = 2^n - 1 entries per feature.
   std::vector<float> binThresholds;
   int32_t binTableDepth = 0;
