@@ -583,27 +583,34 @@ __device__ __forceinline__ void BinSearchRows(const float (&v)[kBinRowsPerPass],
 template <int kLevels> // search depth: the table holds 2^kLevels - 1 thresholds per feature
 __global__ void __launch_bounds__(kBinWaves * 64)
 BinRowsKernel(const float *__restrict__ x, const float *__restrict__ table, uint8_t *__restrict__ ranks,
-              int64_t rows, int F, int rowBlocksPerBlock) {
+              int64_t rows, int F, int rowBlocksPerBlock, int chunks) {
   extern __shared__ __align__(16) unsigned char lds[];
   typedef uint32_t Piece __attribute__((ext_vector_type(4)));
   static_assert(kBinRows == 4 * kBinRowsPerPass, "four passes per row block");
+  // Workgroups go to the 8 XCDs in turn, each with its own L2.  A row is not aligned to cache lines
+  // (F * 4 bytes is no multiple of 128 in general), so neighbouring feature chunks of the same rows
+  // share lines: blocks 8 apart in launch order (same XCD, back to back) take neighbouring chunks of
+  // one group of row blocks, and the shared lines are fetched from HBM once.
+  const uint32_t linear = blockIdx.x;
+  const int chunk = (int)((linear >> 3) % (uint32_t)chunks);
+  const int64_t rowGroup = (int64_t)(linear & 7u) + 8 * (int64_t)(linear / (8u * (uint32_t)chunks));
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int f0 = blockIdx.x * kBinFeatures;
+  const int f0 = chunk * kBinFeatures;
   const int f = f0 + lane;
   constexpr int depth = (1 << kLevels) - 1;
   constexpr uint32_t tableBytes = (uint32_t)depth * kBinFeatures * 4u;
   {
     float *tab = reinterpret_cast<float *>(lds);
-    const float *src = table + (int64_t)blockIdx.x * depth * kBinFeatures;
+    const float *src = table + (int64_t)chunk * depth * kBinFeatures;
     for (int i = tid; i < depth * kBinFeatures; i += kBinWaves * 64) tab[i] = src[i];
   }
   __syncthreads(); // the only block-wide barrier: from here on the waves run on their own
   unsigned char *stage = lds + tableBytes + (uint32_t)wave * (64u * kBinLaneStride);
   unsigned char *mine = stage + lane * kBinLaneStride;
   const int64_t numRowBlocks = (rows + kBinRows - 1) / kBinRows;
-  const int64_t rbBegin = (int64_t)blockIdx.y * rowBlocksPerBlock;
+  const int64_t rbBegin = rowGroup * rowBlocksPerBlock; // (past the end for the padding blocks of the last 8 groups)
   const int64_t rbEnd = rbBegin + rowBlocksPerBlock < numRowBlocks ? rbBegin + rowBlocksPerBlock : numRowBlocks;
   const int fClamped = f < F ? f : F - 1;
   const uint32_t laneBytes = (uint32_t)lane * 4u;
@@ -854,15 +861,17 @@ hipError_t LaunchBinRows(const float *x, const float *table, uint8_t *ranks, int
   int64_t perBlock = (rowBlocks * chunks + 2047) / 2048;
   if (perBlock < kBinWaves) perBlock = kBinWaves;
   if (perBlock > 64 * kBinWaves) perBlock = 64 * kBinWaves;
-  const int64_t gridY = (rowBlocks + perBlock - 1) / perBlock;
-  if (gridY > 65535) return hipErrorInvalidValue;
-  const dim3 grid((unsigned)chunks, (unsigned)gridY), block(kBinWaves * 64);
+  const int64_t rowGroups = (rowBlocks + perBlock - 1) / perBlock;
+  const int64_t blocks = (rowGroups + 7) / 8 * 8 * chunks; // row groups padded to the 8 XCDs
+  if (blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)blocks), block(kBinWaves * 64);
 #define TBAMD_BIN_CASE(LEVELS)                                                                                         \
   case (1 << LEVELS) - 1: {                                                                                            \
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&BinRowsKernel<LEVELS>),                         \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);                    \
     if (e != hipSuccess) return e;                                                                                     \
-    BinRowsKernel<LEVELS><<<grid, block, ldsBytes, stream>>>(x, table, ranks, rows, numFeatures, (int)perBlock);       \
+    BinRowsKernel<LEVELS><<<grid, block, ldsBytes, stream>>>(x, table, ranks, rows, numFeatures, (int)perBlock,       \
+                                                             chunks);                                                  \
     return hipGetLastError();                                                                                          \
   }
   switch (tableDepth) {
