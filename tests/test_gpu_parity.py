@@ -518,3 +518,35 @@ def test_classes_without_trees_score_the_initial_value(tmp_path, kernel):
     runner.run_device_multiclass(dx.data_ptr(), rows, classes.data_ptr(), margins.data_ptr(), None)
     np.testing.assert_allclose(margins.cpu().numpy(), expected, rtol=RTOL_SUM, atol=1e-7)
     np.testing.assert_array_equal(classes.cpu().numpy(), cpu_oracle.argmax_generated(expected))
+
+
+@pytest.mark.parametrize("fine", [False, True], ids=["coarse_thresholds", "fine_thresholds"])
+@pytest.mark.parametrize("features", [1, 2, 63, 130, 257, 600, 1100, 3000, 4500])
+@pytest.mark.parametrize("rows", [200, 3000])
+def test_automatic_plan_over_feature_counts(tmp_path, features, rows, fine):
+    """Whatever kernel the tuner picks for a row width (f32 tile, rank tile, tree-parallel), the answer is the oracle's."""
+    rng = np.random.Generator(np.random.PCG64(features * 7 + rows + fine))
+    grid = np.round(rng.normal(size=(30, features)), 2).astype(np.float32)
+
+    def split():
+        f = int(rng.integers(0, features))
+        if fine and f == 0:
+            return f, rng.normal()                      # feature 0 collects more than 254 distinct thresholds
+        return f, grid[rng.integers(0, 30), f]
+    trees = []
+    for t in range(300 if fine else 60):
+        tree = synth._grow_tree(rng, 6, lambda d, s: 0.85, split, lambda: rng.normal(0.0, 0.2))
+        if fine:
+            tree.feature[0], tree.value[0] = 0, float(np.float32(rng.normal()))
+        trees.append(tree)
+    path = tmp_path / "m.json"
+    synth.write_xgboost_json(path, trees, features)
+    forest = model_io.load_xgboost_json(path)
+    x = np.round(rng.normal(size=(rows, features)), 2).astype(np.float32)
+    runner = make_runner(path, rows)
+    plan = runner.describe_plan()
+    if features in (600, 1100) and rows > 128:            # 64 f32 rows do not fit LDS, 64 rank rows do
+        assert ("quantizedRows=1" in plan) == (not fine), plan
+    if features >= 3000:                                    # not even rank rows fit: a few f32 rows per block
+        assert "kernel=tree_parallel" in plan, plan
+    check_against_oracle(runner, forest, x)
