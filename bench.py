@@ -49,7 +49,11 @@ def main():
     cache = os.path.join(tempfile.gettempdir(), "treebeard_amd_models")
     model = synth.model_path(args.config, cache)
     x = cfg.batch_rows(rows)
-    runner = treebeard.TreebeardInferenceRunner.FromModelFile(model, "", treebeard.CompilerOptions(rows, 1))
+    options = treebeard.CompilerOptions(rows, 1)
+    if cfg.num_class > 0:                       # class ids as int8, the reference's multiclass setting
+        options.SetReturnTypeWidth(8)
+        options.SetReturnTypeIsFloatType(False)
+    runner = treebeard.TreebeardInferenceRunner.FromModelFile(model, "", options)
     multiclass = runner.num_classes() > 0
     dx = torch.from_numpy(x).cuda()
     out = torch.zeros(rows, dtype=torch.int8 if multiclass else torch.float32, device="cuda")

@@ -13,7 +13,9 @@
  *
  * Buffers of the reference entry points are caller-owned HOST memory:
  * inputs  = batchSize x rowSize float32, row-major, contiguous;
- * results = batchSize float32 (int8 class ids for multiclass models).
+ * results = batchSize float32; a multiclass model returns class ids, as int8
+ *           when the options say returnTypeWidth 8 / returnTypeFloatType 0 (what
+ *           the reference's multiclass tests set), as float32 with the default options.
  *
  * The tbmi_ entry points in the second part have no counterpart in the
  * reference: device-resident inference, parity dumps, timing and tuning.
@@ -111,8 +113,10 @@ TBAMD_EXPORT void *findBestGPUScheduleAndCompileModel(void *tbContext);
 TBAMD_EXPORT const char *tbmi_last_error(void);
 TBAMD_EXPORT int32_t tbmi_device_count(void);
 
-/* Inference on rows already resident in device memory (any row count). */
+/* Inference on rows already resident in device memory (any row count); results as RunInference writes them. */
 TBAMD_EXPORT int32_t tbmi_run_device(intptr_t runner, const float *deviceInputs, void *deviceResults, int64_t rows);
+/* Bytes per row that RunInference / tbmi_run_device write: 4 (float32) or 1 (int8 class ids). */
+TBAMD_EXPORT int32_t tbmi_result_bytes(intptr_t runner);
 /* Multiclass: arg-max class ids (int8), per-class sums and softmax (float32 [rows][classes]); any may be null. */
 TBAMD_EXPORT int32_t tbmi_run_device_multiclass(intptr_t runner, const float *deviceInputs, int64_t rows,
                                                 int8_t *deviceClassIds, float *deviceMargins,

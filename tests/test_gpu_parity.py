@@ -33,20 +33,34 @@ def require_gpu():
     assert torch.cuda.is_available()
 
 
-def make_runner(path, batch, kind="xgboost_json", num_features=0, gpu_options=None):
+def make_runner(path, batch, kind="xgboost_json", num_features=0, gpu_options=None, float_class_ids=False):
     options = treebeard.CompilerOptions(batch, 1)
     if num_features:
         options.SetNumberOfFeatures(num_features)
+    if not float_class_ids and is_multiclass(path, kind, num_features):
+        options.SetReturnTypeWidth(8)                  # what the reference's multiclass tests set
+        options.SetReturnTypeIsFloatType(False)        # (test/python/cpu_tests.py:20-22)
     ctx = treebeard.TreebeardContext(str(path), "", options, gpu_options)
     ctx.SetInputFiletype(kind)
     ctx.SetRepresentationType("gpu_sparse")
     return treebeard.TreebeardInferenceRunner.GPUInferenceRunnerFromTBContext(ctx)
 
 
+def is_multiclass(path, kind, num_features):
+    lib = api().runtime_lib
+    h = lib.tbmi_load_forest(str(path).encode(), kind.encode(), num_features)
+    assert h, api().last_error()
+    info = (ctypes.c_int64 * 6)()
+    initial = ctypes.c_double()
+    assert lib.tbmi_forest_info(h, info, ctypes.byref(initial)) == 0
+    lib.tbmi_delete_forest(h)
+    return info[2] > 0
+
+
 def gpu_predict(runner, x):
     dx = torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).cuda()
     rows = x.shape[0]
-    if runner.num_classes() > 0:
+    if runner.result_dtype() == np.int8:
         out = torch.full((rows,), -1, dtype=torch.int8, device="cuda")
     else:
         out = torch.full((rows,), float("nan"), dtype=torch.float32, device="cuda")
@@ -370,7 +384,7 @@ def test_host_buffer_entry_point_pipelines_large_batches(synth_model, k, rows):
     x = synth.CONFIGS[k].batch_rows(rows, seed_offset=2)
     runner = make_runner(synth_model(k), rows)
     device = gpu_predict(runner, x)
-    host = runner.RunInference(x, resultType=np.int8 if runner.num_classes() > 0 else np.float32)
+    host = runner.RunInference(x, resultType=runner.result_dtype())
     np.testing.assert_array_equal(host, device)
     forest = model_io.load_xgboost_json(synth_model(k))
     pick = np.random.default_rng(k).choice(rows, size=2048, replace=False)
@@ -550,3 +564,30 @@ def test_automatic_plan_over_feature_counts(tmp_path, features, rows, fine):
     if features >= 3000:                                    # not even rank rows fit: a few f32 rows per block
         assert "kernel=tree_parallel" in plan, plan
     check_against_oracle(runner, forest, x)
+
+
+def test_multiclass_return_type_follows_the_options(synth_model, tmp_path):
+    """Default options (32-bit float results) return the class id as float32, the reference's multiclass
+    setting (returnTypeWidth 8, not float) as int8; through the host-buffer entry point as well, and a
+    compiled-model file keeps the choice."""
+    rows = 700
+    forest = model_io.load_xgboost_json(synth_model(3))
+    x = synth.CONFIGS[3].batch_rows(rows, seed_offset=8)
+    expected, _ = cpu_oracle.predict(forest, x)
+    as_float = make_runner(synth_model(3), rows, float_class_ids=True)
+    dx = torch.from_numpy(x).cuda()
+    out = torch.full((rows,), float("nan"), dtype=torch.float32, device="cuda")
+    as_float.run_device(dx.data_ptr(), out.data_ptr(), rows)
+    np.testing.assert_array_equal(out.cpu().numpy(), expected)
+    np.testing.assert_array_equal(as_float.RunInference(x, np.float32), expected)
+    as_int8 = make_runner(synth_model(3), rows)
+    np.testing.assert_array_equal(as_int8.RunInference(x, np.int8), expected.astype(np.int8))
+    for runner, dtype in ((as_float, np.float32), (as_int8, np.int8)):
+        path = str(tmp_path / ("m_%s.tbamd" % np.dtype(dtype).name))
+        runner.save_compiled_model(path)
+        reopened = treebeard.TreebeardInferenceRunner.FromCompiledModelFile(path)
+        np.testing.assert_array_equal(reopened.RunInference(x, dtype), expected.astype(dtype))
+    options = treebeard.CompilerOptions(rows, 1)
+    options.SetReturnTypeWidth(16)
+    with pytest.raises(RuntimeError, match="8-bit integers or 32-bit floats"):
+        treebeard.TreebeardInferenceRunner.FromModelFile(synth_model(3), "", options)

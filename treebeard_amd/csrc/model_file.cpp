@@ -21,7 +21,7 @@ namespace tbamd {
 namespace {
 
 constexpr char kMagic[8] = {'T', 'B', 'A', 'M', 'D', 'M', 'D', 'L'};
-constexpr uint32_t kVersion = 1;
+constexpr uint32_t kVersion = 2;
 
 struct Writer {
   std::string bytes;
@@ -54,11 +54,14 @@ struct Reader {
 
 } // namespace
 
-void SaveCompiledModel(const std::string &path, const Forest &forest, const LaunchPlan &plan, int32_t batchSize) {
+void SaveCompiledModel(const std::string &path, const Forest &forest, const LaunchPlan &plan, int32_t batchSize,
+                       int32_t returnTypeWidth, bool returnTypeFloatType) {
   Writer w;
   w.bytes.append(kMagic, sizeof(kMagic));
   w.Put<uint32_t>(kVersion);
   w.Put<int32_t>(batchSize);
+  w.Put<int32_t>(returnTypeWidth);
+  w.Put<int32_t>(returnTypeFloatType ? 1 : 0);
   w.Put<int32_t>(forest.numFeatures);
   w.Put<double>(forest.initialValue);
   w.Put<int32_t>((int32_t)forest.transform);
@@ -95,6 +98,8 @@ CompiledModel LoadCompiledModel(const std::string &path) {
   if (r.Get<uint32_t>() != kVersion) throw Error("unsupported compiled model version");
   CompiledModel m;
   m.batchSize = r.Get<int32_t>();
+  m.returnTypeWidth = r.Get<int32_t>();
+  m.returnTypeFloatType = r.Get<int32_t>() != 0;
   m.forest.numFeatures = r.Get<int32_t>();
   m.forest.initialValue = r.Get<double>();
   m.forest.transform = (Transform)r.Get<int32_t>();

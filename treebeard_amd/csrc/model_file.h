@@ -12,9 +12,12 @@ struct CompiledModel {
   Forest forest;
   LaunchPlan plan;
   int32_t batchSize = 0;
+  int32_t returnTypeWidth = 32;
+  bool returnTypeFloatType = true;
 };
 
-void SaveCompiledModel(const std::string &path, const Forest &forest, const LaunchPlan &plan, int32_t batchSize);
+void SaveCompiledModel(const std::string &path, const Forest &forest, const LaunchPlan &plan, int32_t batchSize,
+                       int32_t returnTypeWidth, bool returnTypeFloatType);
 CompiledModel LoadCompiledModel(const std::string &path);
 
 // Leaf hit counts of a profiling run (the reference's probability profile), with the counts of the

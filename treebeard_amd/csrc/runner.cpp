@@ -43,8 +43,11 @@ void InferenceRunner::InitDevice() {
   if (m_options.batchSize <= 0) throw Error("batchSize must be positive");
   if (m_options.inputElementTypeWidth != 32) throw Error("only 32-bit float inputs are supported");
   if (m_options.thresholdTypeWidth != 32) throw Error("only 32-bit float thresholds are supported");
-  if (m_forest.numClasses == 0 && (m_options.returnTypeWidth != 32 || !m_options.returnTypeFloatType))
-    throw Error("only 32-bit float predictions are supported");
+  const bool floatResults = m_options.returnTypeWidth == 32 && m_options.returnTypeFloatType;
+  const bool int8Results = m_options.returnTypeWidth == 8 && !m_options.returnTypeFloatType;
+  if (m_forest.numClasses == 0 && !floatResults) throw Error("only 32-bit float predictions are supported");
+  if (m_forest.numClasses > 0 && !floatResults && !int8Results)
+    throw Error("class ids are returned as 8-bit integers or 32-bit floats");
   m_forest.Validate();
 
   int deviceCount = 0;
@@ -225,7 +228,7 @@ void InferenceRunner::RunDevice(const float *deviceInputs, void *deviceResults, 
   const int runs = gMeasureGpuKernelTime ? std::max(1, gNumberOfKernelRuns) : 1;
   if (gMeasureGpuKernelTime) Check(hipEventRecord(m_evStart, m_stream), "hipEventRecord");
   for (int i = 0; i < runs; ++i) {
-    if (m_forest.numClasses > 0)
+    if (ClassIdsAsInt8())
       Launch(deviceInputs, rows, nullptr, static_cast<int8_t *>(deviceResults), nullptr, nullptr, nullptr);
     else
       Launch(deviceInputs, rows, static_cast<float *>(deviceResults), nullptr, nullptr, nullptr, nullptr);
@@ -265,7 +268,6 @@ void InferenceRunner::RunInference(const void *hostInputs, void *hostResults) {
   EnsureStaging();
   const int64_t rows = m_options.batchSize;
   const size_t rowBytes = (size_t)m_forest.numFeatures * sizeof(float);
-  const bool multiclass = m_forest.numClasses > 0;
   // Large batches go through in pieces: the copy of piece i+1 (on its own stream) overlaps the kernels
   // of piece i.  Rows are independent, so the pieces give the same results as one launch.
   constexpr int kMaxPieces = 8;
@@ -290,7 +292,7 @@ void InferenceRunner::RunInference(const void *hostInputs, void *hostResults) {
             "copy inputs");
       Check(hipEventRecord(m_pieceReady[p], m_copyStream), "hipEventRecord");
       Check(hipStreamWaitEvent(m_stream, m_pieceReady[p], 0), "hipStreamWaitEvent");
-      if (multiclass)
+      if (ClassIdsAsInt8())
         Launch(dIn, count, nullptr, static_cast<int8_t *>(m_dStageOut) + first, nullptr, nullptr, nullptr);
       else
         Launch(dIn, count, static_cast<float *>(m_dStageOut) + first, nullptr, nullptr, nullptr, nullptr);
@@ -335,7 +337,7 @@ void InferenceRunner::TimeKernels(const float *deviceInputs, void *deviceResults
     f.treeSlices = m_model.PartialCount();
     f.initialValue = m_forest.initialValue;
     f.transform = p.s.transform;
-    if (m_forest.numClasses > 0) f.classOut = static_cast<int8_t *>(deviceResults);
+    if (ClassIdsAsInt8()) f.classOut = static_cast<int8_t *>(deviceResults);
     else f.out = static_cast<float *>(deviceResults);
     Check(hipEventRecord(m_evStart, m_stream), "hipEventRecord");
     for (int i = 0; i < runs; ++i) Check(LaunchFinalize(f, m_stream), "launch finalize kernel");

@@ -56,7 +56,11 @@ public:
   int32_t RowSize() const { return m_forest.numFeatures; }
   int32_t NumTrees() const { return (int32_t)m_forest.trees.size(); }
   int32_t NumClasses() const { return m_forest.numClasses; }
-  int32_t ReturnTypeBytes() const { return m_forest.numClasses > 0 ? 1 : 4; }
+  // Regressors and binary classifiers return float32; multiclass models return the class id as int8
+  // (returnTypeWidth 8, the reference's multiclass setting) or as float32 (its default options).
+  bool ClassIdsAsInt8() const { return m_forest.numClasses > 0 && m_options.returnTypeWidth == 8; }
+  int32_t ReturnTypeBytes() const { return ClassIdsAsInt8() ? 1 : 4; }
+  const CompilerOptions &Options() const { return m_options; }
   int64_t LastKernelMicros() const { return m_lastKernelMicros; }
   const PackedModel &Model() const { return m_model; }
   const Forest &GetForest() const { return m_forest; }

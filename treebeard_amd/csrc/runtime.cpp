@@ -318,6 +318,8 @@ int32_t tbmi_run_device(intptr_t h, const float *in, void *out, int64_t rows) {
   return Guard([&] { Runner(h)->RunDevice(in, out, rows); return 0; }, -1);
 }
 
+int32_t tbmi_result_bytes(intptr_t h) { return Guard([&] { return Runner(h)->ReturnTypeBytes(); }, -1); }
+
 int32_t tbmi_run_device_multiclass(intptr_t h, const float *in, int64_t rows, int8_t *cls, float *margins,
                                    float *probs) {
   return Guard([&] { Runner(h)->RunDeviceMulticlass(in, rows, cls, margins, probs); return 0; }, -1);
@@ -435,7 +437,8 @@ int32_t tbmi_save_compiled_model(intptr_t h, const char *path) {
   return Guard(
       [&] {
         InferenceRunner *r = Runner(h);
-        SaveCompiledModel(path ? path : "", r->GetForest(), r->Model().plan, r->BatchSize());
+        SaveCompiledModel(path ? path : "", r->GetForest(), r->Model().plan, r->BatchSize(),
+                          r->Options().returnTypeWidth, r->Options().returnTypeFloatType);
         return 0;
       },
       -1);
@@ -447,6 +450,8 @@ intptr_t tbmi_load_compiled_model(const char *path, int32_t batchSize) {
         CompiledModel m = LoadCompiledModel(path ? path : "");
         CompilerOptions options;
         options.batchSize = batchSize > 0 ? batchSize : m.batchSize;
+        options.returnTypeWidth = m.returnTypeWidth;
+        options.returnTypeFloatType = m.returnTypeFloatType;
         return reinterpret_cast<intptr_t>(new InferenceRunner(std::move(m.forest), options, m.plan));
       },
       0);

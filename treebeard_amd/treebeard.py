@@ -249,6 +249,7 @@ class TreebeardInferenceRunner:
     def RunInference(self, inputs, resultType=numpy.float32):
         inputs = self._host_inputs(inputs)
         assert inputs.size == self.batchSize * self.rowSize, "RunInference takes exactly one batch"
+        self._check_result_type(resultType)
         results = numpy.zeros((self.batchSize,), resultType)
         _lib().RunInference(self.inferenceRunner, inputs.ctypes.data, results.ctypes.data)
         if api().last_error():
@@ -259,6 +260,7 @@ class TreebeardInferenceRunner:
         inputs = self._host_inputs(inputs)
         numRows = inputs.shape[0]
         assert numRows % self.batchSize == 0
+        self._check_result_type(resultType)
         results = numpy.zeros((numRows,), resultType)
         _lib().RunInferenceOnMultipleBatches(self.inferenceRunner, inputs.ctypes.data, results.ctypes.data, numRows)
         if api().last_error():
@@ -305,6 +307,16 @@ class TreebeardInferenceRunner:
                                           ctypes.byref(walk), ctypes.byref(fin), ctypes.byref(pre)),
                  "tbmi_time_kernels")
         return walk.value, fin.value, pre.value
+
+    def _check_result_type(self, resultType):
+        # the library writes result_dtype() elements: a narrower numpy buffer would be overrun
+        if numpy.dtype(resultType).itemsize != numpy.dtype(self.result_dtype()).itemsize:
+            raise ValueError("this runner returns %s results (see CompilerOptions.SetReturnTypeWidth), not %s"
+                             % (numpy.dtype(self.result_dtype()).name, numpy.dtype(resultType).name))
+
+    def result_dtype(self):
+        """numpy dtype of the results RunInference / run_device write for this runner."""
+        return numpy.int8 if _lib().tbmi_result_bytes(self.inferenceRunner) == 1 else numpy.float32
 
     def set_global_walk_plan(self, rows_per_block=256, interleave=4, tree_slices=1):
         self._rc(_lib().tbmi_set_global_walk_plan(self.inferenceRunner, rows_per_block, interleave, tree_slices),
