@@ -591,3 +591,43 @@ def test_multiclass_return_type_follows_the_options(synth_model, tmp_path):
     options.SetReturnTypeWidth(16)
     with pytest.raises(RuntimeError, match="8-bit integers or 32-bit floats"):
         treebeard.TreebeardInferenceRunner.FromModelFile(synth_model(3), "", options)
+
+
+# The option sets of the reference's GPU auto-schedule tests (test/python/gpu_tests.py:260-325): batch 200,
+# 20 rows per thread block, with and without unrolling / interleaving / tree threads, under each of its
+# three GPU representation names, fed in fixed batches and compared with the model's golden CSV
+# (test/python/test_utils.py:140-166).
+REFERENCE_AUTO_SCHEDULES = {
+    "no-cache": dict(rows_per_thread=2, unroll=False, tree_threads=1, interleave=0),
+    "no-cache-unroll": dict(rows_per_thread=2, unroll=True, tree_threads=1, interleave=0),
+    "unroll-treepar": dict(rows_per_thread=2, unroll=True, tree_threads=4, interleave=0),
+    "unroll-interleave-treepar": dict(rows_per_thread=1, unroll=True, tree_threads=4, interleave=2),
+}
+
+
+@pytest.mark.parametrize("representation", ["gpu_array", "gpu_sparse", "gpu_reorg"])
+@pytest.mark.parametrize("schedule", sorted(REFERENCE_AUTO_SCHEDULES))
+@pytest.mark.parametrize("name", BENCHMARK_XGB)
+def test_reference_auto_schedule_matrix(name, schedule, representation, plain_file):
+    cfg = REFERENCE_AUTO_SCHEDULES[schedule]
+    x, expected = model_io.read_csv(benchmark_csv(name))
+    x = x.astype(np.float32)
+    gpu = treebeard.GPUAutoScheduleOptions()
+    gpu.NumberOfRowsPerThreadBlock(20)
+    gpu.NumberOfRowsPerThread(cfg["rows_per_thread"])
+    gpu.UnrollTreeWalks(cfg["unroll"])
+    gpu.CacheRows(False)
+    gpu.CacheTrees(False)
+    gpu.NumberOfTreeThreads(cfg["tree_threads"])
+    gpu.NumberOfTreesAtATime(1)
+    if cfg["interleave"]:
+        gpu.TreeWalkInterleaveFactor(cfg["interleave"])
+    batch = 100                                           # the fixture CSVs hold 200 rows: two batches
+    ctx = treebeard.TreebeardContext(plain_file(benchmark_model(name)), "", treebeard.CompilerOptions(batch, 1),
+                                     gpuAutoScheduleOptions=gpu)
+    ctx.SetRepresentationType(representation)
+    ctx.SetInputFiletype("xgboost_json")
+    runner = treebeard.TreebeardInferenceRunner.GPUInferenceRunnerFromTBContext(ctx)
+    for first in range(0, x.shape[0], batch):
+        got = runner.RunInference(x[first:first + batch], np.float32)
+        np.testing.assert_allclose(got, expected[first:first + batch], rtol=RTOL_SUM, atol=ATOL_PROB)
