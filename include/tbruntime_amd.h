@@ -115,6 +115,9 @@ TBAMD_EXPORT int32_t tbmi_device_count(void);
 
 /* Inference on rows already resident in device memory (any row count); results as RunInference writes them. */
 TBAMD_EXPORT int32_t tbmi_run_device(intptr_t runner, const float *deviceInputs, void *deviceResults, int64_t rows);
+/* Host buffers like RunInference, but any number of rows (the reference fixes the batch at compile time,
+ * src/runtime/runtime.cpp:58-67): batch-sized windows, copies overlapped with the kernels. */
+TBAMD_EXPORT int32_t tbmi_run_host(intptr_t runner, const void *hostInputs, void *hostResults, int64_t rows);
 /* Bytes per row that RunInference / tbmi_run_device write: 4 (float32) or 1 (int8 class ids). */
 TBAMD_EXPORT int32_t tbmi_result_bytes(intptr_t runner);
 /* Multiclass: arg-max class ids (int8), per-class sums and softmax (float32 [rows][classes]); any may be null. */

@@ -631,3 +631,15 @@ def test_reference_auto_schedule_matrix(name, schedule, representation, plain_fi
     for first in range(0, x.shape[0], batch):
         got = runner.RunInference(x[first:first + batch], np.float32)
         np.testing.assert_allclose(got, expected[first:first + batch], rtol=RTOL_SUM, atol=ATOL_PROB)
+
+
+@pytest.mark.parametrize("k,batch,rows", [(1, 256, 1000), (2, 4096, 4096 * 2 + 77), (3, 1000, 2999), (2, 1 << 18, (1 << 18) + 5)])
+def test_host_entry_point_takes_any_number_of_rows(synth_model, k, batch, rows):
+    """The reference fixes the batch at compile time; tbmi_run_host walks longer (or shorter) host inputs in
+    batch-sized windows and must give the bits of one device-resident launch."""
+    x = synth.CONFIGS[k].batch_rows(rows, seed_offset=12)
+    runner = make_runner(synth_model(k), batch)
+    expected = gpu_predict(runner, x)
+    np.testing.assert_array_equal(runner.run_host(x), expected)
+    np.testing.assert_array_equal(runner.run_host(x[:batch // 3]), expected[:batch // 3])
+    assert runner.run_host(x[:0]).shape == (0,)

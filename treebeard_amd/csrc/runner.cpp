@@ -265,8 +265,23 @@ void InferenceRunner::DumpLeafIds(const float *deviceInputs, int32_t *deviceLeaf
 }
 
 void InferenceRunner::RunInference(const void *hostInputs, void *hostResults) {
+  RunHostChunk(hostInputs, hostResults, m_options.batchSize);
+}
+
+void InferenceRunner::RunHost(const void *hostInputs, void *hostResults, int64_t rows) {
+  if (rows < 0) throw Error("negative row count");
+  if (rows > 0 && (!hostInputs || !hostResults)) throw Error("null host buffer");
+  // the staging buffers hold one compiled batch: longer inputs go through in batch-sized windows
+  const int64_t window = m_options.batchSize;
+  const size_t rowBytes = (size_t)m_forest.numFeatures * sizeof(float);
+  for (int64_t first = 0; first < rows; first += window)
+    RunHostChunk(static_cast<const char *>(hostInputs) + (size_t)first * rowBytes,
+                 static_cast<char *>(hostResults) + (size_t)first * ReturnTypeBytes(), std::min(window, rows - first));
+}
+
+void InferenceRunner::RunHostChunk(const void *hostInputs, void *hostResults, int64_t rows) {
+  if (rows <= 0) return;
   EnsureStaging();
-  const int64_t rows = m_options.batchSize;
   const size_t rowBytes = (size_t)m_forest.numFeatures * sizeof(float);
   // Large batches go through in pieces: the copy of piece i+1 (on its own stream) overlaps the kernels
   // of piece i.  Rows are independent, so the pieces give the same results as one launch.

@@ -35,7 +35,9 @@ public:
 
   // Host buffers, exactly batchSize rows (src/runtime/runtime.cpp:58-67).
   void RunInference(const void *hostInputs, void *hostResults);
-  // Device-resident rows; `out` is f32[rows] (int8[rows] for multiclass models).
+  // Host buffers, any number of rows: batch-sized windows, each copied and computed in overlapping pieces.
+  void RunHost(const void *hostInputs, void *hostResults, int64_t rows);
+  // Device-resident rows; `out` holds ReturnTypeBytes() per row.
   void RunDevice(const float *deviceInputs, void *deviceResults, int64_t rows);
   // Multiclass extras: any of the outputs may be null.
   void RunDeviceMulticlass(const float *deviceInputs, int64_t rows, int8_t *classIds, float *margins,
@@ -68,6 +70,7 @@ public:
   hipStream_t Stream() const { return m_stream; }
 
 private:
+  void RunHostChunk(const void *hostInputs, void *hostResults, int64_t rows); // rows <= batchSize
   void InitDevice();
   void UploadModel();
   void FreeModel();

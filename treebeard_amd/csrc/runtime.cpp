@@ -318,6 +318,15 @@ int32_t tbmi_run_device(intptr_t h, const float *in, void *out, int64_t rows) {
   return Guard([&] { Runner(h)->RunDevice(in, out, rows); return 0; }, -1);
 }
 
+int32_t tbmi_run_host(intptr_t h, const void *in, void *out, int64_t rows) {
+  return Guard(
+      [&] {
+        Runner(h)->RunHost(in, out, rows);
+        return 0;
+      },
+      -1);
+}
+
 int32_t tbmi_result_bytes(intptr_t h) { return Guard([&] { return Runner(h)->ReturnTypeBytes(); }, -1); }
 
 int32_t tbmi_run_device_multiclass(intptr_t h, const float *in, int64_t rows, int8_t *cls, float *margins,

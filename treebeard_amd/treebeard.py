@@ -308,6 +308,15 @@ class TreebeardInferenceRunner:
                  "tbmi_time_kernels")
         return walk.value, fin.value, pre.value
 
+    def run_host(self, inputs):
+        """Any number of host rows (numpy in, numpy out); the batch size only sizes the staging buffers."""
+        inputs = self._host_inputs(inputs)
+        rows = inputs.size // self.rowSize
+        assert rows * self.rowSize == inputs.size
+        results = numpy.zeros((rows,), self.result_dtype())
+        self._rc(_lib().tbmi_run_host(self.inferenceRunner, inputs.ctypes.data, results.ctypes.data, rows), "tbmi_run_host")
+        return results
+
     def _check_result_type(self, resultType):
         # the library writes result_dtype() elements: a narrower numpy buffer would be overrun
         if numpy.dtype(resultType).itemsize != numpy.dtype(self.result_dtype()).itemsize:
