@@ -80,6 +80,12 @@ def check_against_oracle(runner, forest, x):
     pred, sums = cpu_oracle.predict(forest, x)
     got = gpu_predict(runner, x)
     if forest.num_classes > 0:
+        voted = np.isin(np.arange(forest.num_classes), forest.class_id)
+        if not voted.all():
+            # a class without trees scores the initial value, as in the reference's generated code
+            # (test_classes_without_trees_score_the_initial_value states the two reference behaviours)
+            margins = np.where(voted[None, :], sums, forest.initial_value).astype(np.float32)
+            pred = cpu_oracle.argmax_generated(margins).astype(np.float32)
         np.testing.assert_array_equal(got.astype(np.float32), pred)
     elif forest.transform == model_io.SIGMOID:
         np.testing.assert_allclose(got, pred, rtol=0, atol=ATOL_PROB)
@@ -643,3 +649,57 @@ def test_host_entry_point_takes_any_number_of_rows(synth_model, k, batch, rows):
     np.testing.assert_array_equal(runner.run_host(x), expected)
     np.testing.assert_array_equal(runner.run_host(x[:batch // 3]), expected[:batch // 3])
     assert runner.run_host(x[:0]).shape == (0,)
+
+
+def _random_forest_file(rng, path):
+    features = int(rng.choice([1, 2, 5, 17, 40, 100, 300]))
+    num_class = int(rng.choice([0, 0, 0, 3, 7]))
+    depth = int(rng.integers(0, 11))
+    trees_n = int(rng.choice([1, 2, 9, 40, 150]))
+    split_p = float(rng.choice([0.5, 0.8, 1.0])) if depth <= 8 else 0.6
+    lopsided = rng.random() < 0.3
+    prob = (lambda d, s: (0.95 if s <= 0 else 0.2)) if lopsided else (lambda d, s: split_p)
+    grid = np.round(rng.normal(size=(25, features)), 1).astype(np.float32)
+    trees = [synth._grow_tree(rng, depth, prob, lambda: (lambda f: (f, grid[rng.integers(0, 25), f]))(int(rng.integers(0, features))),
+                              lambda: rng.normal(0.0, 0.3), force_root=bool(rng.random() < 0.8)) for _ in range(trees_n)]
+    objective = "multi:softmax" if num_class else str(rng.choice(["reg:squarederror", "binary:logistic"]))
+    info = [int(c) for c in rng.permutation(trees_n) % num_class] if num_class else None
+    synth.write_xgboost_json(path, trees, features, objective=objective, num_class=num_class, tree_info=info,
+                             base_score=str(rng.choice(["5E-1", "2.5E-1", "0.7"])))
+    return features
+
+
+@pytest.mark.parametrize("seed", range(200))
+def test_random_forests_and_plans(tmp_path, seed):
+    """Differential run over random shapes: model, batch size, launch options; leaf ids and predictions vs the oracle."""
+    rng = np.random.Generator(np.random.PCG64(9000 + seed))
+    path = tmp_path / "m.json"
+    features = _random_forest_file(rng, path)
+    forest = model_io.load_xgboost_json(path)
+    rows = int(rng.choice([1, 2, 33, 64, 129, 500, 2049, 9000]))
+    x = np.round(rng.normal(size=(rows, features)), 1).astype(np.float32)      # many values sit on thresholds
+    x[rng.random(x.shape) < 0.01] = np.inf
+    x[rng.random(x.shape) < 0.01] = -np.inf
+    gpu = None
+    if rng.random() < 0.5:
+        gpu = treebeard.GPUAutoScheduleOptions.Construct(num_rows_per_TB=int(rng.choice([8, 20, 64, 128, 256, 512])),
+                                                         num_tree_threads=int(rng.choice([1, 2, 4, 10])))
+        gpu.TreeWalkInterleaveFactor(int(rng.choice([1, 2, 4, 8])))
+    runner = make_runner(path, rows, gpu_options=gpu)
+    check_against_oracle(runner, forest, x)
+    kind = rng.integers(0, 4)
+    try:
+        if kind == 0:
+            runner.set_global_walk_plan(int(rng.choice([64, 256, 1024])), int(rng.choice([1, 2, 4, 8])), int(rng.integers(1, 50)))
+        elif kind == 1:
+            runner.set_quantized_plan(int(rng.choice([1, 4, 16])), int(rng.choice([1, 2, 4])), 0, int(rng.integers(1, 6)))
+        elif kind == 2:
+            lanes = int(rng.choice([1, 4, 16, 64, 256]))
+            runner.set_tree_parallel_plan(max(1, 256 // lanes) if lanes < 256 else int(rng.choice([1, 2, 4])), lanes,
+                                          int(rng.choice([1, 2, 4])), 0, int(rng.integers(0, 9)))
+        else:
+            rb = int(rng.choice([64, 128, 256]))
+            runner.set_plan(rb, int(rng.choice([1, 2, 4])), int(rng.choice([1, 2, 4, 8])), 0, int(rng.integers(0, 9)))
+    except RuntimeError:
+        pass                                              # a plan this model does not fit: refused, runner unchanged
+    check_against_oracle(runner, forest, x)

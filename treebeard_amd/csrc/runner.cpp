@@ -116,6 +116,8 @@ void InferenceRunner::UploadModel() {
 
 void InferenceRunner::Repack(const LaunchPlan &plan) {
   PackedModel next = PackForest(m_forest, plan);
+  // refuse before anything is freed: a plan that fails leaves the runner as it was
+  if (next.LdsBytes() > (size_t)m_limits.ldsBytesPerBlock) throw Error("launch plan exceeds the LDS of one workgroup");
   Check(hipStreamSynchronize(m_stream), "hipStreamSynchronize");
   FreeModel();
   m_model = std::move(next);
