@@ -40,7 +40,7 @@ struct WalkParams {
 };
 
 struct FinalizeParams {
-  const double *partial = nullptr; // [slices][rows][max(1, classes)]
+  double *partial = nullptr;   // [slices][rows][max(1, classes)]; the wide finalize parks class sums in slice 0
   int64_t rows = 0;
   int32_t numClasses = 0;
   int32_t treeSlices = 1;      // number of partial sums per (row, class)

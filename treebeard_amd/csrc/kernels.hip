@@ -713,7 +713,7 @@ __global__ void __launch_bounds__(256) FinalizeWideKernel(const FinalizeParams p
     return;
   }
   // classifiers: park the class sum in the first slice's slot; FinalizeKernel (1 slice) does the rest
-  if (lane == 0) const_cast<double *>(p.partial)[row * Cn + c] = margin - p.initialValue;
+  if (lane == 0) p.partial[row * Cn + c] = margin - p.initialValue;
 }
 
 template <int K, int PF, int W>
