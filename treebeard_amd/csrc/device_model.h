@@ -66,6 +66,9 @@ struct DeviceGroup {
   uint32_t nodeCount;   // multiple of 2 so that the group is a whole number of 16-byte pieces
   uint32_t bundleBegin;
   uint32_t bundleCount;
+  uint32_t uniformClass; // class id + 1 when every bundle of the group votes for one class, else 0
+  uint32_t reserved[3];
 };
+static_assert(sizeof(DeviceGroup) == 32, "group descriptors are fetched with one 32-byte scalar load");
 
 } // namespace tbamd

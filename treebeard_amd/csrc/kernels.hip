@@ -235,13 +235,16 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
     while (b0 < grp.bundleCount) {
       uint32_t b1 = grp.bundleCount;
       if (C > 0) {
-        const int cls = (int)bundles[grp.bundleBegin + b0].classId;
+        // most groups vote for one class: the descriptor says so and no bundle has to be looked at
+        const int cls = grp.uniformClass ? (int)grp.uniformClass - 1 : (int)bundles[grp.bundleBegin + b0].classId;
         if (cls != curClass) { // classes arrive in ascending order
           TBAMD_FLUSH_CLASS(cls)
           curClass = cls;
         }
-        b1 = b0 + 1;
-        while (b1 < grp.bundleCount && (int)bundles[grp.bundleBegin + b1].classId == cls) ++b1;
+        if (!grp.uniformClass) {
+          b1 = b0 + 1;
+          while (b1 < grp.bundleCount && (int)bundles[grp.bundleBegin + b1].classId == cls) ++b1;
+        }
       }
       for (uint32_t b = b0 + tt; b < b1; b += TT) {
         const DeviceBundle bd = bundles[grp.bundleBegin + b];

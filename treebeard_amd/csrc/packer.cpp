@@ -225,6 +225,13 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
     }
     g.nodeCount = (uint32_t)pm.nodes.size() - g.nodeBegin;
     g.bundleCount = (uint32_t)pm.bundles.size() - g.bundleBegin;
+    g.uniformClass = 0;
+    if (g.bundleCount > 0) {
+      const uint32_t first = pm.bundles[g.bundleBegin].classId;
+      bool uniform = true;
+      for (uint32_t b = 1; b < g.bundleCount; ++b) uniform = uniform && pm.bundles[g.bundleBegin + b].classId == first;
+      if (uniform) g.uniformClass = first + 1;
+    }
     pm.maxGroupNodes = std::max(pm.maxGroupNodes, g.nodeCount);
   };
 
