@@ -133,6 +133,7 @@ def main():
                      "kernel": ("BinRowsKernel+" if quantized else "") + kernel,
                      "kernel_ms": walk_ms, "finalize_ms": fin_ms, "bin_ms": bin_ms,
                      "algorithmic_bytes_per_row": hbm_bytes_row,
+                     "binding": binding,       # which memory roofline binds this workload: see roofline_binding
                      "measured_copy_gbs": copy_gbs,
                      "frac_of_measured_copy": hbm_gbs / copy_gbs if copy_gbs else None},
         "roofline_binding": {"bound": binding, "achieved": lds_gbs if binding == "lds" else hbm_gbs,
