@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtreebeard_amd.so")
 SOURCES = ["forest.cpp", "json_reader.cpp", "xgboost_loader.cpp", "onnx_loader.cpp", "packer.cpp", "tuner.cpp", "model_file.cpp",
-           "runner.cpp", "runtime.cpp", "kernels.hip"]
+           "host_copy.cpp", "runner.cpp", "runtime.cpp", "kernels.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -69,6 +69,8 @@ InferenceRunner::~InferenceRunner() {
   (void)hipFree(m_dRanks);
   (void)hipFree(m_dStageIn);
   (void)hipFree(m_dStageOut);
+  for (void *buf : m_pinned)
+    if (buf) (void)hipHostFree(buf);
   for (auto &ev : m_pieceReady)
     if (ev) (void)hipEventDestroy(ev);
   if (m_copyStream) (void)hipStreamDestroy(m_copyStream);
@@ -281,32 +283,67 @@ void InferenceRunner::RunHost(const void *hostInputs, void *hostResults, int64_t
                  static_cast<char *>(hostResults) + (size_t)first * ReturnTypeBytes(), std::min(window, rows - first));
 }
 
+namespace {
+
+// True when the runtime knows the address as pinned (or registered) host memory, which DMA reads
+// directly; pageable memory makes the query fail, and that error must not linger.
+bool IsPinnedHost(const void *ptr) {
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, ptr) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return attr.type == hipMemoryTypeHost;
+}
+
+} // namespace
+
 void InferenceRunner::RunHostChunk(const void *hostInputs, void *hostResults, int64_t rows) {
   if (rows <= 0) return;
   EnsureStaging();
   const size_t rowBytes = (size_t)m_forest.numFeatures * sizeof(float);
+  const size_t totalBytes = (size_t)rows * rowBytes;
   // Large batches go through in pieces: the copy of piece i+1 (on its own stream) overlaps the kernels
   // of piece i.  Rows are independent, so the pieces give the same results as one launch.
-  constexpr int kMaxPieces = 8;
-  int pieces = 1;
-  if (!gMeasureGpuKernelTime && (size_t)rows * rowBytes >= ((size_t)16 << 20))
-    pieces = (int)std::min<int64_t>(kMaxPieces, rows / 4096);
-  if (pieces <= 1) {
-    Check(hipMemcpyAsync(m_dStageIn, hostInputs, (size_t)rows * rowBytes, hipMemcpyHostToDevice, m_stream), "copy inputs");
+  if (gMeasureGpuKernelTime || totalBytes < ((size_t)16 << 20) || rows < 2 * 4096) {
+    Check(hipMemcpyAsync(m_dStageIn, hostInputs, totalBytes, hipMemcpyHostToDevice, m_stream), "copy inputs");
     RunDevice(m_dStageIn, m_dStageOut, rows);
   } else {
     if (!m_copyStream) {
       Check(hipStreamCreateWithFlags(&m_copyStream, hipStreamNonBlocking), "hipStreamCreate");
       for (auto &ev : m_pieceReady) Check(hipEventCreateWithFlags(&ev, hipEventDisableTiming), "hipEventCreate");
     }
+    // Pinned inputs are read by DMA where they lie, in 8 pieces.  Pageable inputs are first moved into
+    // one of two pinned buffers by a few host threads (one core copies slower than the link carries):
+    // pieces of about 16 MB, the host copy of piece i+1 overlapping the DMA of piece i.
+    const bool staged = !IsPinnedHost(hostInputs);
+    int64_t pieces = staged ? (int64_t)((totalBytes + ((size_t)16 << 20) - 1) >> 24) : 8;
+    pieces = std::max<int64_t>(2, std::min<int64_t>({pieces, (int64_t)kMaxPieces, rows / 4096}));
     const int64_t perPiece = ((rows + pieces - 1) / pieces + 1023) / 1024 * 1024;
+    if (staged) {
+      const size_t pieceBytes = (size_t)perPiece * rowBytes;
+      if (pieceBytes > m_pinnedBytes) {
+        for (void *&buf : m_pinned) {
+          if (buf) (void)hipHostFree(buf);
+          buf = nullptr;
+        }
+        m_pinnedBytes = 0;
+        for (void *&buf : m_pinned) Check(hipHostMalloc(&buf, pieceBytes, hipHostMallocDefault), "allocate pinned staging");
+        m_pinnedBytes = pieceBytes;
+      }
+      if (!m_copier) m_copier.reset(new ParallelCopier((int)std::min(8u, std::max(1u, std::thread::hardware_concurrency()))));
+    }
     int p = 0;
     for (int64_t first = 0; first < rows; first += perPiece, ++p) {
       const int64_t count = std::min(perPiece, rows - first);
       float *dIn = m_dStageIn + first * m_forest.numFeatures;
-      Check(hipMemcpyAsync(dIn, static_cast<const char *>(hostInputs) + (size_t)first * rowBytes, (size_t)count * rowBytes,
-                           hipMemcpyHostToDevice, m_copyStream),
-            "copy inputs");
+      const char *src = static_cast<const char *>(hostInputs) + (size_t)first * rowBytes;
+      if (staged) {
+        if (p >= 2) Check(hipEventSynchronize(m_pieceReady[p - 2]), "hipEventSynchronize"); // its buffer is free again
+        m_copier->Copy(m_pinned[p & 1], src, (size_t)count * rowBytes);
+        src = static_cast<const char *>(m_pinned[p & 1]);
+      }
+      Check(hipMemcpyAsync(dIn, src, (size_t)count * rowBytes, hipMemcpyHostToDevice, m_copyStream), "copy inputs");
       Check(hipEventRecord(m_pieceReady[p], m_copyStream), "hipEventRecord");
       Check(hipStreamWaitEvent(m_stream, m_pieceReady[p], 0), "hipStreamWaitEvent");
       if (ClassIdsAsInt8())

@@ -10,11 +10,13 @@
 #include "forest.h"
 #include "kernels.h"
 #include "options.h"
+#include "host_copy.h"
 #include "packer.h"
 #include "tuner.h"
 
 #include <hip/hip_runtime.h>
 
+#include <memory>
 #include <string>
 
 namespace tbamd {
@@ -91,7 +93,12 @@ private:
   PackedModel m_model;
   hipStream_t m_stream = nullptr;
   hipStream_t m_copyStream = nullptr; // host-buffer entry point: copies of the next piece overlap the kernels
-  hipEvent_t m_pieceReady[8] = {};
+  static constexpr int kMaxPieces = 64;
+  hipEvent_t m_pieceReady[kMaxPieces] = {};
+  // pageable inputs pass through two pinned buffers, filled by a few host threads
+  void *m_pinned[2] = {nullptr, nullptr};
+  size_t m_pinnedBytes = 0;
+  std::unique_ptr<ParallelCopier> m_copier;
   hipEvent_t m_evStart = nullptr, m_evStop = nullptr;
 
   DeviceGlobalNode *m_dGlobalNodes = nullptr;
