@@ -390,8 +390,11 @@ def test_host_buffer_entry_point_pipelines_large_batches(synth_model, k, rows):
     x = synth.CONFIGS[k].batch_rows(rows, seed_offset=2)
     runner = make_runner(synth_model(k), rows)
     device = gpu_predict(runner, x)
-    host = runner.RunInference(x, resultType=runner.result_dtype())
+    host = runner.RunInference(x, resultType=runner.result_dtype())              # pageable: staged through pinned buffers
     np.testing.assert_array_equal(host, device)
+    np.testing.assert_array_equal(runner.RunInference(x, resultType=runner.result_dtype()), device)   # buffers reused
+    pinned = torch.from_numpy(x).pin_memory()                                        # pinned: read by DMA where it lies
+    np.testing.assert_array_equal(runner.RunInference(pinned.numpy(), resultType=runner.result_dtype()), device)
     forest = model_io.load_xgboost_json(synth_model(k))
     pick = np.random.default_rng(k).choice(rows, size=2048, replace=False)
     pred, _ = cpu_oracle.predict(forest, x[pick])
