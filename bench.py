@@ -66,6 +66,7 @@ def main():
         b.copy_(a)
         torch.cuda.synchronize()
 
+    torch.cuda.synchronize()                    # buffers ready before the runner's own stream reads them
     for _ in range(args.warmup):
         runner.run_device(dx.data_ptr(), out.data_ptr(), rows)
     torch.cuda.synchronize()

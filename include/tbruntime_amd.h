@@ -113,7 +113,10 @@ TBAMD_EXPORT void *findBestGPUScheduleAndCompileModel(void *tbContext);
 TBAMD_EXPORT const char *tbmi_last_error(void);
 TBAMD_EXPORT int32_t tbmi_device_count(void);
 
-/* Inference on rows already resident in device memory (any row count); results as RunInference writes them. */
+/* Inference on rows already resident in device memory (any row count); results as RunInference writes them.
+ * The kernels run on a stream of the runner that does not order itself with any other stream: whatever
+ * produced the buffers (a fill, a copy, a kernel on the caller's stream) must have completed before the
+ * call - synchronise that stream first.  The call returns after the results are written. */
 TBAMD_EXPORT int32_t tbmi_run_device(intptr_t runner, const float *deviceInputs, void *deviceResults, int64_t rows);
 /* Host buffers like RunInference, but any number of rows (the reference fixes the batch at compile time,
  * src/runtime/runtime.cpp:58-67): batch-sized windows, copies overlapped with the kernels. */

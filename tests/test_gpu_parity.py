@@ -64,6 +64,7 @@ def gpu_predict(runner, x):
         out = torch.full((rows,), -1, dtype=torch.int8, device="cuda")
     else:
         out = torch.full((rows,), float("nan"), dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()      # the library does not wait for other streams: buffers must be ready
     runner.run_device(dx.data_ptr(), out.data_ptr(), rows)
     return out.cpu().numpy()
 
@@ -71,6 +72,7 @@ def gpu_predict(runner, x):
 def gpu_leaf_ids(runner, x):
     dx = torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).cuda()
     ids = torch.full((x.shape[0], runner.num_trees()), -7, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()      # the library does not wait for other streams: buffers must be ready
     runner.dump_leaf_ids(dx.data_ptr(), ids.data_ptr(), x.shape[0])
     return ids.cpu().numpy()
 
@@ -165,6 +167,7 @@ def test_synthetic_configurations(synth_model, k, rows):
         cls = torch.zeros(rows, dtype=torch.int8, device="cuda")
         margins = torch.zeros((rows, 8), dtype=torch.float32, device="cuda")
         probs = torch.zeros((rows, 8), dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()      # the library does not wait for other streams: buffers must be ready
         runner.run_device_multiclass(dx.data_ptr(), rows, cls.data_ptr(), margins.data_ptr(), probs.data_ptr())
         pred, sums = cpu_oracle.predict(forest, x)
         np.testing.assert_allclose(margins.cpu().numpy(), sums, rtol=RTOL_SUM, atol=1e-7)
@@ -329,6 +332,7 @@ def test_degenerate_models(tmp_path):
 
 def test_zero_rows_and_errors(synth_model):
     runner = make_runner(synth_model(1), 16)
+    torch.cuda.synchronize()      # the library does not wait for other streams: buffers must be ready
     runner.run_device(None, None, 0)
     lib = api().runtime_lib
     assert lib.tbmi_run_device(0, None, None, 4) == -1 and "null" in api().last_error()
@@ -357,6 +361,7 @@ def test_kernel_time_shim(synth_model):
     assert ten > one > 0
     dx = torch.from_numpy(x).cuda()
     out = torch.zeros(1024, dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()      # the library does not wait for other streams: buffers must be ready
     walk_ms, fin_ms = runner.time_kernels(dx.data_ptr(), out.data_ptr(), 1024, 5)
     assert 0 < walk_ms < 50 and fin_ms >= 0
 
@@ -380,6 +385,7 @@ def test_row_staging_alignment_and_ragged_tails(tmp_path, rows, features, offset
         runner = make_runner(path, rows)
         setup(runner)
         out.fill_(float("nan"))
+        torch.cuda.synchronize()      # the library does not wait for other streams: buffers must be ready
         runner.run_device(flat.data_ptr() + 4 * offset, out.data_ptr(), rows)
         np.testing.assert_allclose(out.cpu().numpy(), expected, rtol=RTOL_SUM, atol=0)
 
@@ -461,6 +467,7 @@ def test_many_tree_slices_on_small_batches(synth_model, k, rows, slices):
     if k == 3:
         dx = torch.from_numpy(x).cuda()
         margins = torch.zeros((rows, 8), dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()      # the library does not wait for other streams: buffers must be ready
         runner.run_device_multiclass(dx.data_ptr(), rows, None, margins.data_ptr(), None)
         np.testing.assert_allclose(margins.cpu().numpy(), cpu_oracle.predict(forest, x)[1], rtol=RTOL_SUM, atol=1e-7)
 
@@ -538,6 +545,7 @@ def test_classes_without_trees_score_the_initial_value(tmp_path, kernel):
     dx = torch.from_numpy(x).cuda()
     margins = torch.zeros((rows, 7), dtype=torch.float32, device="cuda")
     classes = torch.zeros((rows,), dtype=torch.int8, device="cuda")
+    torch.cuda.synchronize()      # the library does not wait for other streams: buffers must be ready
     runner.run_device_multiclass(dx.data_ptr(), rows, classes.data_ptr(), margins.data_ptr(), None)
     np.testing.assert_allclose(margins.cpu().numpy(), expected, rtol=RTOL_SUM, atol=1e-7)
     np.testing.assert_array_equal(classes.cpu().numpy(), cpu_oracle.argmax_generated(expected))
@@ -586,6 +594,7 @@ def test_multiclass_return_type_follows_the_options(synth_model, tmp_path):
     as_float = make_runner(synth_model(3), rows, float_class_ids=True)
     dx = torch.from_numpy(x).cuda()
     out = torch.full((rows,), float("nan"), dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()      # the library does not wait for other streams: buffers must be ready
     as_float.run_device(dx.data_ptr(), out.data_ptr(), rows)
     np.testing.assert_array_equal(out.cpu().numpy(), expected)
     np.testing.assert_array_equal(as_float.RunInference(x, np.float32), expected)
@@ -642,7 +651,8 @@ def test_reference_auto_schedule_matrix(name, schedule, representation, plain_fi
         np.testing.assert_allclose(got, expected[first:first + batch], rtol=RTOL_SUM, atol=ATOL_PROB)
 
 
-@pytest.mark.parametrize("k,batch,rows", [(1, 256, 1000), (2, 4096, 4096 * 2 + 77), (3, 1000, 2999), (2, 1 << 18, (1 << 18) + 5)])
+@pytest.mark.parametrize("k,batch,rows", [(1, 256, 1000), (2, 4096, 4096 * 2 + 77), (3, 1000, 2999), (2, 1 << 18, (1 << 18) + 5),
+                                          (1, 64, 64 * 5000 + 3), (4, 512, 512 * 70)])
 def test_host_entry_point_takes_any_number_of_rows(synth_model, k, batch, rows):
     """The reference fixes the batch at compile time; tbmi_run_host walks longer (or shorter) host inputs in
     batch-sized windows and must give the bits of one device-resident launch."""
@@ -652,6 +662,8 @@ def test_host_entry_point_takes_any_number_of_rows(synth_model, k, batch, rows):
     np.testing.assert_array_equal(runner.run_host(x), expected)
     np.testing.assert_array_equal(runner.run_host(x[:batch // 3]), expected[:batch // 3])
     assert runner.run_host(x[:0]).shape == (0,)
+    whole = rows // batch * batch
+    np.testing.assert_array_equal(runner.RunInferenceOnMultipleBatches(x[:whole], runner.result_dtype()), expected[:whole])
 
 
 def _random_forest_file(rng, path):

@@ -159,11 +159,17 @@ const float *InferenceRunner::PrepareRows(const float *deviceInputs, int64_t row
   return reinterpret_cast<const float *>(m_dRanks);
 }
 
-void InferenceRunner::EnsureStaging() {
-  if (m_dStageIn) return;
-  const size_t rows = (size_t)m_options.batchSize;
-  Check(hipMalloc(reinterpret_cast<void **>(&m_dStageIn), rows * m_forest.numFeatures * sizeof(float)), "allocate input staging");
-  Check(hipMalloc(&m_dStageOut, rows * sizeof(float)), "allocate output staging");
+void InferenceRunner::EnsureStaging(int64_t rows) {
+  if (rows <= m_stageRows) return;
+  Check(hipStreamSynchronize(m_stream), "hipStreamSynchronize");
+  (void)hipFree(m_dStageIn);
+  (void)hipFree(m_dStageOut);
+  m_dStageIn = nullptr;
+  m_dStageOut = nullptr;
+  m_stageRows = 0;
+  Check(hipMalloc(reinterpret_cast<void **>(&m_dStageIn), (size_t)rows * m_forest.numFeatures * sizeof(float)), "allocate input staging");
+  Check(hipMalloc(&m_dStageOut, (size_t)rows * sizeof(float)), "allocate output staging");
+  m_stageRows = rows;
 }
 
 hipError_t InferenceRunner::LaunchWalk(const WalkParams &p) const {
@@ -275,9 +281,11 @@ void InferenceRunner::RunInference(const void *hostInputs, void *hostResults) {
 void InferenceRunner::RunHost(const void *hostInputs, void *hostResults, int64_t rows) {
   if (rows < 0) throw Error("negative row count");
   if (rows > 0 && (!hostInputs || !hostResults)) throw Error("null host buffer");
-  // the staging buffers hold one compiled batch: longer inputs go through in batch-sized windows
-  const int64_t window = m_options.batchSize;
+  // Windows of at least one compiled batch and at most about 256 MB of rows (the staging buffers grow
+  // to the window): a long input of small batches is not walked one small batch at a time.
   const size_t rowBytes = (size_t)m_forest.numFeatures * sizeof(float);
+  const int64_t cap = std::max<int64_t>(m_options.batchSize, (int64_t)(((size_t)256 << 20) / rowBytes));
+  const int64_t window = std::min<int64_t>(cap, std::max<int64_t>(rows, 1));
   for (int64_t first = 0; first < rows; first += window)
     RunHostChunk(static_cast<const char *>(hostInputs) + (size_t)first * rowBytes,
                  static_cast<char *>(hostResults) + (size_t)first * ReturnTypeBytes(), std::min(window, rows - first));
@@ -300,7 +308,7 @@ bool IsPinnedHost(const void *ptr) {
 
 void InferenceRunner::RunHostChunk(const void *hostInputs, void *hostResults, int64_t rows) {
   if (rows <= 0) return;
-  EnsureStaging();
+  EnsureStaging(rows);
   const size_t rowBytes = (size_t)m_forest.numFeatures * sizeof(float);
   const size_t totalBytes = (size_t)rows * rowBytes;
   // Large batches go through in pieces: the copy of piece i+1 (on its own stream) overlaps the kernels

@@ -72,12 +72,12 @@ public:
   hipStream_t Stream() const { return m_stream; }
 
 private:
-  void RunHostChunk(const void *hostInputs, void *hostResults, int64_t rows); // rows <= batchSize
+  void RunHostChunk(const void *hostInputs, void *hostResults, int64_t rows);
   void InitDevice();
   void UploadModel();
   void FreeModel();
   void EnsurePartial(int64_t rows);
-  void EnsureStaging();
+  void EnsureStaging(int64_t rows);
   void EnsureRanks(int64_t rows);
   // Rank-quantised plans: runs the binning kernel and returns the buffer the walk kernel reads.
   const float *PrepareRows(const float *deviceInputs, int64_t rows);
@@ -115,6 +115,7 @@ private:
   size_t m_ranksBytes = 0;
   float *m_dStageIn = nullptr;
   void *m_dStageOut = nullptr;
+  int64_t m_stageRows = 0;
   int64_t m_lastKernelMicros = 0;
 };
 

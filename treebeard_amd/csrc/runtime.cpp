@@ -117,11 +117,9 @@ void RunInference(intptr_t h, void *inputs, void *results) {
 void RunInferenceOnMultipleBatches(intptr_t h, void *inputs, void *results, int32_t numRows) {
   GuardVoid([&] {
     InferenceRunner *r = Runner(h);
-    const int32_t batch = r->BatchSize();
-    if (numRows % batch != 0) throw Error("numRows must be a multiple of the batch size");
-    for (int32_t b = 0; b < numRows / batch; ++b)
-      r->RunInference(static_cast<char *>(inputs) + (size_t)b * batch * r->RowSize() * sizeof(float),
-                      static_cast<char *>(results) + (size_t)b * batch * r->ReturnTypeBytes());
+    if (numRows % r->BatchSize() != 0) throw Error("numRows must be a multiple of the batch size");
+    // rows are independent: the batches go through together (same results as one RunInference per batch)
+    r->RunHost(inputs, results, numRows);
   });
 }
 
