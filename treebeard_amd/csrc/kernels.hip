@@ -719,17 +719,23 @@ __global__ void __launch_bounds__(256) FinalizeWideKernel(const FinalizeParams p
   if (lane == 0) p.partial[row * Cn + c] = margin - p.initialValue;
 }
 
+// The ceiling on dynamic LDS is an attribute of each kernel: it is raised once per kernel, to the whole
+// 160 KB, instead of on every launch (a runtime call that small batches would pay for each time).
+template <auto Kernel> hipError_t AllowFullLds() {
+  static const hipError_t status =
+      hipFuncSetAttribute(reinterpret_cast<const void *>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  return status;
+}
+
 template <int K, int PF, int W>
 hipError_t LaunchWalkKP(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
   if (p.leafIds) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&WalkRowsLdsKernel<K, PF, W, true>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
+    hipError_t e = AllowFullLds<&WalkRowsLdsKernel<K, PF, W, true>>();
     if (e != hipSuccess) return e;
     WalkRowsLdsKernel<K, PF, W, true><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out,
                                                                          p.partial, p.leafIds, p.nodeOrigin, p.slotTree);
   } else {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&WalkRowsLdsKernel<K, PF, W, false>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
+    hipError_t e = AllowFullLds<&WalkRowsLdsKernel<K, PF, W, false>>();
     if (e != hipSuccess) return e;
     WalkRowsLdsKernel<K, PF, W, false><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out,
                                                                           p.partial, nullptr, nullptr, nullptr);
@@ -782,14 +788,12 @@ namespace {
 template <int K, int PF>
 hipError_t LaunchTreeParallelKP(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
   if (p.leafIds) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&WalkTreeParallelKernel<K, PF, true>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
+    hipError_t e = AllowFullLds<&WalkTreeParallelKernel<K, PF, true>>();
     if (e != hipSuccess) return e;
     WalkTreeParallelKernel<K, PF, true><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out,
                                                                           p.partial, p.leafIds, p.nodeOrigin, p.slotTree);
   } else {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&WalkTreeParallelKernel<K, PF, false>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);
+    hipError_t e = AllowFullLds<&WalkTreeParallelKernel<K, PF, false>>();
     if (e != hipSuccess) return e;
     WalkTreeParallelKernel<K, PF, false><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out,
                                                                            p.partial, nullptr, nullptr, nullptr);
@@ -870,8 +874,7 @@ hipError_t LaunchBinRows(const float *x, const float *table, uint8_t *ranks, int
   const dim3 grid((unsigned)blocks), block(kBinWaves * 64);
 #define TBAMD_BIN_CASE(LEVELS)                                                                                         \
   case (1 << LEVELS) - 1: {                                                                                            \
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&BinRowsKernel<LEVELS>),                         \
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes);                    \
+    hipError_t e = AllowFullLds<&BinRowsKernel<LEVELS>>();                                                             \
     if (e != hipSuccess) return e;                                                                                     \
     BinRowsKernel<LEVELS><<<grid, block, ldsBytes, stream>>>(x, table, ranks, rows, numFeatures, (int)perBlock,       \
                                                              chunks);                                                  \
