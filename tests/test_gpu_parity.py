@@ -188,7 +188,7 @@ def test_config2_batch_sweep(synth_model, rows):
         np.testing.assert_allclose(gpu_predict(runner, x), pred, rtol=0, atol=ATOL_PROB)
 
 
-@pytest.mark.parametrize("k", [2, 3, 5])
+@pytest.mark.parametrize("k", [2, 3, 5, 4])
 def test_full_size_properties(synth_model, k):
     cfg = synth.CONFIGS[k]
     rows = cfg.batch
