@@ -237,3 +237,23 @@ def test_hit_count_profile_agrees_with_oracle_walks(lib, tmp_path, synth_model):
     assert lib.tbmi_forest_load_profile(h, str(path).encode(), ctypes.byref(rows), ctypes.byref(steps)) == 0, last_error()
     assert rows.value == 500 and abs(steps.value - plen.sum() / 500) < 1e-9
     lib.tbmi_delete_forest(h)
+
+
+def test_c_client_builds_against_the_header_and_sees_documented_errors(tmp_path, synth_model):
+    """The public header is plain C; a C99 program links the library and meets the documented error behaviour
+    (0 / -1 and a message, never an abort; no CPU fallback when there is no device)."""
+    import shutil
+    import subprocess
+    from treebeard_amd.runtime_api import LIB_PATH
+    if shutil.which("gcc") is None:
+        pytest.skip("needs gcc")
+    root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..")
+    exe = str(tmp_path / "abi_client")
+    libdir = os.path.dirname(LIB_PATH)
+    build = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(root, "include"),
+                            os.path.join(root, "tests", "native", "abi_client.c"), "-L", libdir, "-ltreebeard_amd",
+                            "-Wl,-rpath," + libdir, "-o", exe], capture_output=True, text=True)
+    assert build.returncode == 0, build.stderr
+    run = subprocess.run([exe, synth_model(1)], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0, (run.returncode, run.stdout, run.stderr)
+    assert "trees=100 features=8 classes=0" in run.stdout
