@@ -27,16 +27,26 @@ template <typename T> T *Upload(const std::vector<T> &host, const char *what) {
 InferenceRunner::InferenceRunner(Forest forest, const CompilerOptions &options,
                                  const GPUAutoScheduleOptions *gpuOptions)
     : m_forest(std::move(forest)), m_options(options) {
-  InitDevice();
-  m_model = PackForest(m_forest, ChoosePlan(m_forest, m_options.batchSize, gpuOptions, m_limits));
-  UploadModel();
+  try {
+    InitDevice();
+    m_model = PackForest(m_forest, ChoosePlan(m_forest, m_options.batchSize, gpuOptions, m_limits));
+    UploadModel();
+  } catch (...) { // a constructor that throws gets no destructor call: give back what was created
+    Release();
+    throw;
+  }
 }
 
 InferenceRunner::InferenceRunner(Forest forest, const CompilerOptions &options, const LaunchPlan &plan)
     : m_forest(std::move(forest)), m_options(options) {
-  InitDevice();
-  m_model = PackForest(m_forest, plan);
-  UploadModel();
+  try {
+    InitDevice();
+    m_model = PackForest(m_forest, plan);
+    UploadModel();
+  } catch (...) {
+    Release();
+    throw;
+  }
 }
 
 void InferenceRunner::InitDevice() {
@@ -62,7 +72,9 @@ void InferenceRunner::InitDevice() {
   Check(hipEventCreate(&m_evStop), "hipEventCreate");
 }
 
-InferenceRunner::~InferenceRunner() {
+InferenceRunner::~InferenceRunner() { Release(); }
+
+void InferenceRunner::Release() noexcept {
   if (m_stream) (void)hipStreamSynchronize(m_stream);
   FreeModel();
   (void)hipFree(m_dPartial);

@@ -72,6 +72,7 @@ public:
   hipStream_t Stream() const { return m_stream; }
 
 private:
+  void Release() noexcept;
   void RunHostChunk(const void *hostInputs, void *hostResults, int64_t rows);
   void InitDevice();
   void UploadModel();
