@@ -116,6 +116,30 @@ def main():
         torch.cuda.synchronize()
         copy_gbs = 5 * 2 * (1 << 30) / (ev0.elapsed_time(ev1) * 1e-3) / 1e9
         del src, dst
+    # ... and the LDS: conflict-free reads of 4, 8 and 16 bytes per lane on every CU (the library's micro-benchmark)
+    lds_measured = None
+    if not args.copy_calibration:
+        import ctypes
+        from treebeard_amd.runtime_api import api
+        lds_measured = {}
+        for width in (4, 8, 16):
+            rate = ctypes.c_double()
+            if api().runtime_lib.tbmi_lds_read_bandwidth(width, ctypes.byref(rate)) != 0:
+                sys.exit("bench.py: " + api().last_error())
+            lds_measured["b%d" % (8 * width)] = rate.value / 1e9
+    # What the LDS pipes need at those measured rates for this kernel's own mix (an 8-byte node read and a 4-byte
+    # feature read per level, a 4-byte leaf read per tree): for the visited nodes only, and for the lock-step walk
+    # that takes every row through the depth of each tree (the depth of the deepest tree of a bundle, in fact).
+    lds_floor = None
+    if lds_measured and binding == "lds":
+        per_level = 8.0 / (lds_measured["b64"] * 1e9) + 4.0 / (lds_measured["b32"] * 1e9)
+        per_leaf = 4.0 / (lds_measured["b32"] * 1e9)
+        depth_sum = float(sum(forest.depth(t) for t in range(forest.num_trees)))
+        visited_ms = rows * (steps_per_row * per_level + forest.num_trees * per_leaf) * 1e3
+        lockstep_ms = rows * (depth_sum * per_level + forest.num_trees * per_leaf) * 1e3
+        lds_floor = {"visited_nodes_ms": visited_ms, "frac_of_visited_floor": visited_ms / walk_ms,
+                     "lockstep_levels_per_row": depth_sum, "lockstep_ms": lockstep_ms,
+                     "frac_of_lockstep_floor": lockstep_ms / walk_ms}
     traffic = None
     traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(traffic_file):
@@ -143,6 +167,9 @@ def main():
                              "kernel": kernel, "kernel_ms": walk_ms, "path_ms": path_ms,
                              "algorithmic_bytes_per_row": lds_bytes_row if binding == "lds" else hbm_bytes_row,
                              "visited_nodes_per_row": steps_per_row,
+                             "measured_lds_read_gbs": lds_measured,
+                             "lds_floor": lds_floor,
+                             "frac_of_measured_lds": (lds_gbs / lds_measured["b128"]) if (lds_measured and binding == "lds") else None,
                              "peak_note": "LDS: 256 CUs x 256 B/clk x 2.4 GHz (ds_read_b128 measured 237 B/clk/CU); "
                                           "a scalar walk moves 10 B per lane per two LDS instructions (4 clk), so "
                                           "62.5 % is its ceiling"},

@@ -67,5 +67,7 @@ hipError_t LaunchWalkTreeParallel(const WalkParams &p, int interleave, size_t ld
 // one per row; p.globalNodes / p.globalTrees instead of groups and bundles.
 hipError_t LaunchWalkGlobal(const WalkParams &p, int interleave, hipStream_t stream);
 hipError_t LaunchFinalize(const FinalizeParams &p, hipStream_t stream);
+// Conflict-free LDS reads of 4, 8 or 16 bytes per lane on every CU: the measured bytes per second.
+hipError_t MeasureLdsReadBandwidth(int widthBytes, int computeUnits, hipStream_t stream, double *bytesPerSecond);
 
 } // namespace tbamd

@@ -58,6 +58,7 @@ SIGNATURES = {
     "tbmi_time_kernels": (c_i32, [c_ip, c_vp, c_vp, c_i64, c_i32, ctypes.POINTER(ctypes.c_double),
                                   ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]),
     "tbmi_result_bytes": (c_i32, [c_ip]),
+    "tbmi_lds_read_bandwidth": (c_i32, [c_i32, ctypes.POINTER(ctypes.c_double)]),
     "tbmi_run_host": (c_i32, [c_ip, c_vp, c_vp, c_i64]),
     "tbmi_set_global_walk_plan": (c_i32, [c_ip, c_i32, c_i32, c_i32]),
     "tbmi_set_quantized_plan": (c_i32, [c_ip, c_i32, c_i32, c_i32, c_i32]),
