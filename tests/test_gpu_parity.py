@@ -718,3 +718,14 @@ def test_random_forests_and_plans(tmp_path, seed):
     except RuntimeError:
         pass                                              # a plan this model does not fit: refused, runner unchanged
     check_against_oracle(runner, forest, x)
+
+
+def test_lds_micro_benchmark_reports_plausible_rates():
+    lib = api().runtime_lib
+    rates = {}
+    for width in (4, 8, 16):
+        rate = ctypes.c_double()
+        assert lib.tbmi_lds_read_bandwidth(width, ctypes.byref(rate)) == 0, api().last_error()
+        rates[width] = rate.value
+    assert 1e13 < rates[4] < rates[8] <= 1.3 * rates[16] < 4e14          # tens to hundreds of TB/s on 256 CUs
+    assert lib.tbmi_lds_read_bandwidth(3, ctypes.byref(ctypes.c_double())) == -1
