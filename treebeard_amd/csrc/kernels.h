@@ -28,6 +28,7 @@ struct WalkParams {
   const float *x = nullptr;       // rows x numFeatures, row-major, device
   const uint4 *nodes16 = nullptr; // packed nodes viewed as 16-byte pieces
   const DeviceBundle *bundles = nullptr;
+  const DeviceNode *bundleRoots = nullptr; // interleave root-node copies per bundle (row-parallel f32 walk)
   const DeviceGroup *groups = nullptr;
   const DeviceGlobalNode *globalNodes = nullptr; // global-memory walk only
   const DeviceGlobalTree *globalTrees = nullptr;

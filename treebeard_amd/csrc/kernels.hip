@@ -117,7 +117,8 @@ __device__ __forceinline__ void StageRows(const float *__restrict__ src, int val
 template <int K, int PF, int kMode, bool kDump>
 __global__ void __launch_bounds__(1024)
 WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16,
-                  const DeviceBundle *__restrict__ bundles, const DeviceGroup *__restrict__ groups,
+                  const DeviceBundle *__restrict__ bundles, const DeviceNode *__restrict__ bundleRoots,
+                  const DeviceGroup *__restrict__ groups,
                   const WalkScalars s, float *__restrict__ out, double *__restrict__ partial,
                   int32_t *__restrict__ leafIds, const int32_t *__restrict__ nodeOrigin,
                   const int32_t *__restrict__ slotTree) {
@@ -252,7 +253,20 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
 #pragma unroll
         for (int k = 0; k < K; ++k) addr[k] = bd.root[k];
         const int depth = (int)bd.depth;
-        for (int d = 0; d < depth; ++d) {
+        // Level 0 of the f32 tiles: copies of the root nodes sit next to the bundles and arrive in scalar
+        // registers, only the feature is read from LDS.  A root that is a leaf holds the walk in place like any other leaf, so the step is safe
+        // for depth 0.  (On rank tiles, whose rounds are latency-bound, the extra scalar load did not pay.)
+        if (kMode != kTileRankU8) {
+          const DeviceNode *roots = bundleRoots + (size_t)(grp.bundleBegin + b) * K;
+#pragma unroll
+          for (int k = 0; k < K; ++k) {
+            const DeviceNode root = roots[k];
+            const uint32_t off = kMode == kTileF32Bytes ? (root.meta & 0xFFFFu) : (root.meta & 0xFFFFu) << 2;
+            const bool left = LdsLoadFloat(column + off) < root.value;
+            addr[k] = (root.meta >> 16) + (left ? 0u : kNodeBytes);
+          }
+        }
+        for (int d = kMode != kTileRankU8 ? 1 : 0; d < depth; ++d) {
 #pragma unroll
           for (int k = 0; k < K; ++k) {
             const U32x2 node = LdsLoadNode(addr[k]);
@@ -732,12 +746,12 @@ hipError_t LaunchWalkKP(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBy
   if (p.leafIds) {
     hipError_t e = AllowFullLds<&WalkRowsLdsKernel<K, PF, W, true>>();
     if (e != hipSuccess) return e;
-    WalkRowsLdsKernel<K, PF, W, true><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out,
+    WalkRowsLdsKernel<K, PF, W, true><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.bundleRoots, p.groups, p.s, p.out,
                                                                          p.partial, p.leafIds, p.nodeOrigin, p.slotTree);
   } else {
     hipError_t e = AllowFullLds<&WalkRowsLdsKernel<K, PF, W, false>>();
     if (e != hipSuccess) return e;
-    WalkRowsLdsKernel<K, PF, W, false><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out,
+    WalkRowsLdsKernel<K, PF, W, false><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.bundleRoots, p.groups, p.s, p.out,
                                                                           p.partial, nullptr, nullptr, nullptr);
   }
   return hipGetLastError();

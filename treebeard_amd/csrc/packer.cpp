@@ -300,6 +300,7 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
           pm.nodeOrigin.push_back(n);
         }
       }
+      for (int k = 0; k < K; ++k) pm.bundleRoots.push_back(pm.nodes[g.nodeBegin + b.root[k] / kNodeBytes]);
       pm.bundles.push_back(b);
       next += count;
       any = true;
@@ -312,6 +313,7 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
       pm.nodeOrigin.resize(marks[keep].nodes);
       pm.slotTree.resize(marks[keep].slots);
       pm.bundles.resize(g.bundleBegin + keep);
+      pm.bundleRoots.resize((size_t)(g.bundleBegin + keep) * K);
       next = marks[keep].next;
     }
     closeGroup();
@@ -321,6 +323,7 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
     openGroup();
     closeGroup();
   }
+  if (pm.bundleRoots.size() != pm.bundles.size() * (size_t)K) throw Error("internal error: bundle root table out of step");
   return pm;
 }
 

@@ -57,6 +57,9 @@ struct PackedModel {
   // Parity/debug side tables (not touched by the timed kernels):
   std::vector<int32_t> nodeOrigin; // per packed node: original node id inside its tree (-1: null leaf)
   std::vector<int32_t> slotTree;   // per bundle slot: original tree index, -1 for a padding tree
+  // Copies of the root nodes, plan.interleave per bundle: every lane of a wave starts a tree at its root, so
+  // the f32 row-parallel walk takes level 0 from scalar registers instead of an LDS node read.
+  std::vector<DeviceNode> bundleRoots;
   uint32_t maxGroupNodes = 0;
   // kGlobalWalk only:
   std::vector<DeviceGlobalNode> globalNodes;

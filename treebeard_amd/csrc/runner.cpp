@@ -94,6 +94,7 @@ void InferenceRunner::Release() noexcept {
 void InferenceRunner::FreeModel() {
   (void)hipFree(m_dNodes);
   (void)hipFree(m_dBundles);
+  (void)hipFree(m_dBundleRoots);
   (void)hipFree(m_dGroups);
   (void)hipFree(m_dNodeOrigin);
   (void)hipFree(m_dSlotTree);
@@ -105,6 +106,7 @@ void InferenceRunner::FreeModel() {
   m_dGlobalTrees = nullptr;
   m_dNodes = nullptr;
   m_dBundles = nullptr;
+  m_dBundleRoots = nullptr;
   m_dGroups = nullptr;
   m_dNodeOrigin = nullptr;
   m_dSlotTree = nullptr;
@@ -122,6 +124,7 @@ void InferenceRunner::UploadModel() {
   if (m_model.LdsBytes() > (size_t)m_limits.ldsBytesPerBlock) throw Error("launch plan exceeds the LDS of one workgroup");
   m_dNodes = Upload(m_model.nodes, "upload nodes");
   m_dBundles = Upload(m_model.bundles, "upload bundles");
+  m_dBundleRoots = Upload(m_model.bundleRoots, "upload bundle roots");
   m_dGroups = Upload(m_model.groups, "upload groups");
   m_dNodeOrigin = Upload(m_model.nodeOrigin, "upload node origins");
   m_dSlotTree = Upload(m_model.slotTree, "upload slot table");
@@ -212,6 +215,7 @@ WalkParams InferenceRunner::MakeWalkParams(const float *deviceInputs, int64_t ro
   p.globalTrees = m_dGlobalTrees;
   p.nodes16 = reinterpret_cast<const uint4 *>(m_dNodes);
   p.bundles = m_dBundles;
+  p.bundleRoots = m_dBundleRoots;
   p.groups = m_dGroups;
   return p;
 }

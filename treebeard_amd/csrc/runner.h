@@ -106,6 +106,7 @@ private:
   DeviceGlobalTree *m_dGlobalTrees = nullptr;
   DeviceNode *m_dNodes = nullptr;
   DeviceBundle *m_dBundles = nullptr;
+  DeviceNode *m_dBundleRoots = nullptr;
   DeviceGroup *m_dGroups = nullptr;
   int32_t *m_dNodeOrigin = nullptr;
   int32_t *m_dSlotTree = nullptr;
