@@ -266,6 +266,7 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
             addr[k] = (root.meta >> 16) + (left ? 0u : kNodeBytes);
           }
         }
+#pragma unroll 2
         for (int d = kMode != kTileRankU8 ? 1 : 0; d < depth; ++d) {
 #pragma unroll
           for (int k = 0; k < K; ++k) {
