@@ -138,7 +138,12 @@ LaunchPlan ChoosePlan(const Forest &forest, int64_t batchSize, const GPUAutoSche
   int32_t rb = 256;
   if (ov && ov->numRowsPerTB > 0) rb = std::max(64, FloorPow2(ov->numRowsPerTB));
   bool words = false;
-  auto fits = [&](int32_t r) { return RowTileFits(forest.numFeatures, r, halfLds + 8192, &words); };
+  // (two blocks per CU only pay while a block keeps 16 KB or more for its tree groups: measured on 56..82
+  //  features, 256 rows win down to 19 KB groups and lose from 15 KB on, where 128 rows x 8 threads take over)
+  auto fits = [&](int32_t r) {
+    const int32_t meetBytes = forest.numClasses > 0 ? r * std::max(1, std::min(8, 1024 / r)) * 8 : 0;
+    return RowTileFits(forest.numFeatures, r, halfLds - meetBytes - 512, &words);
+  };
   while (rb > 64 && !fits(rb)) rb /= 2;
   int32_t budget = halfLds;
   if (!fits(rb)) { // one block per CU
