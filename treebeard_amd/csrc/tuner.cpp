@@ -131,30 +131,48 @@ LaunchPlan ChoosePlan(const Forest &forest, int64_t batchSize, const GPUAutoSche
   LaunchPlan plan;
   plan.kernel = LaunchPlan::Kernel::kRowParallelLds;
 
-  // Shape that measured best on MI355X: blocks of 1024 lanes (16 waves), two blocks per CU
-  // (full occupancy), each block 256 rows x 4 tree threads when the row tile allows it, and the
-  // tree group as large as half the LDS leaves room for.
+  // Block shape, from timings on MI355X (blocks of 1024 lanes; 600-1000 trees of depth 6-8; 28..520 features).
+  // Two blocks per CU hide each other's group loads and barriers, but only while enough LDS is left for
+  // the tree groups; a narrower row tile buys bigger groups; past that one block per CU with the biggest
+  // groups wins.  In order of preference:
+  //   256 rows x 4 tree threads, two blocks per CU, while >= 16 KB remain for a group   (up to ~60 features)
+  //   128 x 8, two blocks, while >= 20 KB remain                                        (up to ~118)
+  //    64 x 16, two blocks, while >= 40 KB remain                                       (up to ~155)
+  //   128 x 8, one block, while >= 56 KB remain                                         (up to ~195)
+  //    64 x 16, one block                                                               (as long as the tile fits)
   const int32_t halfLds = limits.ldsBytesPerBlock / 2;
-  int32_t rb = 256;
-  if (ov && ov->numRowsPerTB > 0) rb = std::max(64, FloorPow2(ov->numRowsPerTB));
   bool words = false;
-  // (two blocks per CU only pay while a block keeps 16 KB or more for its tree groups: measured on 56..82
-  //  features, 256 rows win down to 19 KB groups and lose from 15 KB on, where 128 rows x 8 threads take over)
-  auto fits = [&](int32_t r) {
-    const int32_t meetBytes = forest.numClasses > 0 ? r * std::max(1, std::min(8, 1024 / r)) * 8 : 0;
-    return RowTileFits(forest.numFeatures, r, halfLds - meetBytes - 512, &words);
+  auto treeThreadsFor = [&](int32_t r) {
+    int32_t tt = std::max(1, 1024 / r);
+    if (ov && ov->numTreeThreads > 0) tt = std::max(1, std::min(ov->numTreeThreads, 1024 / r));
+    return tt;
   };
-  while (rb > 64 && !fits(rb)) rb /= 2;
-  int32_t budget = halfLds;
-  if (!fits(rb)) { // one block per CU
-    budget = limits.ldsBytesPerBlock;
-    if (!RowTileFits(forest.numFeatures, rb, budget, &words))
-      throw Error("row tile of " + std::to_string(forest.numFeatures) + " features does not fit LDS");
+  // LDS left for a tree group beside the row tile (and the classifiers' meeting area)
+  auto roomFor = [&](int32_t r, int32_t ldsBytes) -> int64_t {
+    const int64_t tile = (int64_t)(forest.numFeatures + 1) * r * 4;
+    const int64_t meetBytes = forest.numClasses > 0 ? (int64_t)r * treeThreadsFor(r) * 8 : 0;
+    return (int64_t)ldsBytes - tile - meetBytes - 512;
+  };
+  int32_t rb = 64;
+  int32_t budget = limits.ldsBytesPerBlock;
+  if (ov && ov->numRowsPerTB > 0) { // the caller's block shape: two blocks per CU if 16 KB remain, else one
+    rb = std::max(64, FloorPow2(ov->numRowsPerTB));
+    while (rb > 64 && roomFor(rb, limits.ldsBytesPerBlock) < 16384) rb /= 2;
+    if (roomFor(rb, halfLds) >= 16384) budget = halfLds;
+  } else if (roomFor(256, halfLds) >= 16384) {
+    rb = 256, budget = halfLds;
+  } else if (roomFor(128, halfLds) >= 20480) {
+    rb = 128, budget = halfLds;
+  } else if (roomFor(64, halfLds) >= 40960) {
+    rb = 64, budget = halfLds;
+  } else if (roomFor(128, limits.ldsBytesPerBlock) >= 57344) {
+    rb = 128;
   }
+  if (!RowTileFits(forest.numFeatures, rb, budget, &words))
+    throw Error("row tile of " + std::to_string(forest.numFeatures) + " features does not fit LDS");
   plan.rowsPerBlock = rb;
   plan.featureOffsetInWords = words;
-  plan.treeThreads = std::max(1, std::min(8, 1024 / rb));
-  if (ov && ov->numTreeThreads > 0) plan.treeThreads = std::max(1, std::min(ov->numTreeThreads, 1024 / rb));
+  plan.treeThreads = treeThreadsFor(rb);
 
   plan.interleave = 4;
   if (ov && ov->treeWalkInterleaveFactor > 0)
