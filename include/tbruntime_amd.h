@@ -121,6 +121,13 @@ TBAMD_EXPORT int32_t tbmi_lds_read_bandwidth(int32_t widthBytes, double *bytesPe
  * produced the buffers (a fill, a copy, a kernel on the caller's stream) must have completed before the
  * call - synchronise that stream first.  The call returns after the results are written. */
 TBAMD_EXPORT int32_t tbmi_run_device(intptr_t runner, const float *deviceInputs, void *deviceResults, int64_t rows);
+/* The same kernels enqueued on the caller's stream (a hipStream_t; null is the default stream); the call
+ * returns without waiting for them.  Work queued on that stream before the call is seen by the kernels,
+ * work queued after it sees their results: no synchronisation is needed on either side.  The first call,
+ * and a call with more rows than any before it, allocates the runner's partial-sum buffers; while such a
+ * call is made no earlier call on another stream may still be running. */
+TBAMD_EXPORT int32_t tbmi_run_device_async(intptr_t runner, const float *deviceInputs, void *deviceResults,
+                                           int64_t rows, void *stream);
 /* Host buffers like RunInference, but any number of rows (the reference fixes the batch at compile time,
  * src/runtime/runtime.cpp:58-67): batch-sized windows, copies overlapped with the kernels. */
 TBAMD_EXPORT int32_t tbmi_run_host(intptr_t runner, const void *hostInputs, void *hostResults, int64_t rows);

@@ -729,3 +729,29 @@ def test_lds_micro_benchmark_reports_plausible_rates():
         rates[width] = rate.value
     assert 1e13 < rates[4] < rates[8] <= 1.3 * rates[16] < 4e14          # tens to hundreds of TB/s on 256 CUs
     assert lib.tbmi_lds_read_bandwidth(3, ctypes.byref(ctypes.c_double())) == -1
+
+
+@pytest.mark.parametrize("k,rows", [(2, 20000), (3, 9000), (1, 777)])
+def test_async_entry_point_orders_itself_on_the_callers_stream(synth_model, k, rows):
+    """tbmi_run_device_async enqueues on the stream it is handed: inputs produced by work queued on that
+    stream just before the call are seen, results are visible to work queued just after it, and no
+    synchronisation is made on either side (default stream and a side stream)."""
+    forest = model_io.load_xgboost_json(synth_model(k))
+    x = synth.CONFIGS[k].batch_rows(rows, seed_offset=5)
+    runner = make_runner(synth_model(k), rows)
+    expected = gpu_predict(runner, x)
+    host = torch.from_numpy(x).pin_memory()
+    for stream in (torch.cuda.current_stream(), torch.cuda.Stream()):
+        with torch.cuda.stream(stream):
+            dx = torch.empty((rows, x.shape[1]), dtype=torch.float32, device="cuda")
+            out = torch.empty((rows,), dtype=torch.int8 if runner.result_dtype() == np.int8 else torch.float32, device="cuda")
+            for _ in range(3):   # keep the stream busy so that the copy below is still pending at the call
+                dx.normal_()
+            dx.copy_(host, non_blocking=True)
+            runner.run_device_async(dx.data_ptr(), out.data_ptr(), rows, stream.cuda_stream)
+            got = out.to("cpu", non_blocking=False)
+        stream.synchronize()
+        np.testing.assert_array_equal(got.numpy(), expected)
+    pred, _ = cpu_oracle.predict(forest, x)
+    if forest.num_classes == 0:
+        np.testing.assert_allclose(expected, pred, rtol=RTOL_SUM, atol=ATOL_PROB)

@@ -14,14 +14,6 @@ void Check(hipError_t e, const char *what) {
   if (e != hipSuccess) throw Error(std::string(what) + ": " + hipGetErrorString(e));
 }
 
-template <typename T> T *Upload(const std::vector<T> &host, const char *what) {
-  T *ptr = nullptr;
-  const size_t bytes = std::max<size_t>(host.size(), 1) * sizeof(T);
-  Check(hipMalloc(reinterpret_cast<void **>(&ptr), bytes), what);
-  if (!host.empty()) Check(hipMemcpy(ptr, host.data(), host.size() * sizeof(T), hipMemcpyHostToDevice), what);
-  return ptr;
-}
-
 } // namespace
 
 InferenceRunner::InferenceRunner(Forest forest, const CompilerOptions &options,
@@ -141,9 +133,18 @@ void InferenceRunner::Repack(const LaunchPlan &plan) {
   UploadModel();
 }
 
+size_t InferenceRunner::PartialBytes(int64_t rows) const {
+  if (!NeedsFinalize()) return 0;
+  return (size_t)m_model.PartialCount() * (size_t)rows * (size_t)std::max(1, m_forest.numClasses) * sizeof(double);
+}
+
+size_t InferenceRunner::RanksBytes(int64_t rows) const {
+  if (!m_model.plan.quantizedRows) return 0;
+  return (size_t)((rows + 63) / 64) * 64 * (size_t)m_forest.numFeatures;
+}
+
 void InferenceRunner::EnsurePartial(int64_t rows) {
-  if (!NeedsFinalize()) return;
-  const size_t need = (size_t)m_model.PartialCount() * (size_t)rows * (size_t)std::max(1, m_forest.numClasses) * sizeof(double);
+  const size_t need = PartialBytes(rows);
   if (need <= m_partialBytes) return;
   Check(hipStreamSynchronize(m_stream), "hipStreamSynchronize");
   (void)hipFree(m_dPartial);
@@ -154,8 +155,7 @@ void InferenceRunner::EnsurePartial(int64_t rows) {
 }
 
 void InferenceRunner::EnsureRanks(int64_t rows) {
-  if (!m_model.plan.quantizedRows) return;
-  const size_t need = (size_t)((rows + 63) / 64) * 64 * (size_t)m_forest.numFeatures;
+  const size_t need = RanksBytes(rows);
   if (need <= m_ranksBytes) return;
   Check(hipStreamSynchronize(m_stream), "hipStreamSynchronize");
   (void)hipFree(m_dRanks);
@@ -165,13 +165,21 @@ void InferenceRunner::EnsureRanks(int64_t rows) {
   m_ranksBytes = need;
 }
 
-const float *InferenceRunner::PrepareRows(const float *deviceInputs, int64_t rows) {
-  if (!m_model.plan.quantizedRows) return deviceInputs;
+InferenceRunner::Workspace InferenceRunner::OwnWorkspace(int64_t rows) {
+  EnsurePartial(rows);
   EnsureRanks(rows);
-  Check(LaunchBinRows(deviceInputs, m_dBinTable, m_dRanks, rows, m_forest.numFeatures, m_model.binTableDepth,
-                      m_model.binChunkFeatures, m_stream),
+  Workspace ws;
+  ws.partial = m_dPartial;
+  ws.ranks = m_dRanks;
+  return ws;
+}
+
+const float *InferenceRunner::PrepareRows(const float *deviceInputs, int64_t rows, uint8_t *ranks, hipStream_t stream) {
+  if (!m_model.plan.quantizedRows) return deviceInputs;
+  Check(LaunchBinRows(deviceInputs, m_dBinTable, ranks, rows, m_forest.numFeatures, m_model.binTableDepth,
+                      m_model.binChunkFeatures, stream),
         "launch rank-quantisation kernel");
-  return reinterpret_cast<const float *>(m_dRanks);
+  return reinterpret_cast<const float *>(ranks);
 }
 
 void InferenceRunner::EnsureStaging(int64_t rows) {
@@ -187,13 +195,13 @@ void InferenceRunner::EnsureStaging(int64_t rows) {
   m_stageRows = rows;
 }
 
-hipError_t InferenceRunner::LaunchWalk(const WalkParams &p) const {
+hipError_t InferenceRunner::LaunchWalk(const WalkParams &p, hipStream_t stream) const {
   const LaunchPlan &plan = m_model.plan;
-  if (plan.kernel == LaunchPlan::Kernel::kGlobalWalk) return LaunchWalkGlobal(p, plan.interleave, m_stream);
+  if (plan.kernel == LaunchPlan::Kernel::kGlobalWalk) return LaunchWalkGlobal(p, plan.interleave, stream);
   if (plan.kernel == LaunchPlan::Kernel::kTreeParallel)
-    return LaunchWalkTreeParallel(p, plan.interleave, m_model.LdsBytes(), m_stream);
+    return LaunchWalkTreeParallel(p, plan.interleave, m_model.LdsBytes(), stream);
   const int tileMode = plan.quantizedRows ? 2 : (plan.featureOffsetInWords ? 1 : 0);
-  return LaunchWalkRowsLds(p, plan.interleave, tileMode, m_model.LdsBytes(), m_stream);
+  return LaunchWalkRowsLds(p, plan.interleave, tileMode, m_model.LdsBytes(), stream);
 }
 
 WalkParams InferenceRunner::MakeWalkParams(const float *deviceInputs, int64_t rows) const {
@@ -221,22 +229,21 @@ WalkParams InferenceRunner::MakeWalkParams(const float *deviceInputs, int64_t ro
 }
 
 void InferenceRunner::Launch(const float *deviceInputs, int64_t rows, float *out, int8_t *classOut, float *margins,
-                             float *probabilities, int32_t *leafIds) {
+                             float *probabilities, int32_t *leafIds, hipStream_t stream, const Workspace &ws) {
   if (rows <= 0) return;
-  EnsurePartial(rows);
-  WalkParams p = MakeWalkParams(PrepareRows(deviceInputs, rows), rows);
+  WalkParams p = MakeWalkParams(PrepareRows(deviceInputs, rows, ws.ranks, stream), rows);
   const bool finalize = NeedsFinalize();
   p.out = finalize ? nullptr : out;
-  p.partial = finalize ? m_dPartial : nullptr;
+  p.partial = finalize ? ws.partial : nullptr;
   if (leafIds) {
     p.leafIds = leafIds;
     p.nodeOrigin = m_dNodeOrigin;
     p.slotTree = m_dSlotTree;
   }
-  Check(LaunchWalk(p), "launch walk kernel");
+  Check(LaunchWalk(p, stream), "launch walk kernel");
   if (finalize) {
     FinalizeParams f;
-    f.partial = m_dPartial;
+    f.partial = ws.partial;
     f.rows = rows;
     f.numClasses = m_forest.numClasses;
     f.treeSlices = m_model.PartialCount();
@@ -246,18 +253,19 @@ void InferenceRunner::Launch(const float *deviceInputs, int64_t rows, float *out
     f.classOut = classOut;
     f.margins = margins;
     f.probabilities = probabilities;
-    Check(LaunchFinalize(f, m_stream), "launch finalize kernel");
+    Check(LaunchFinalize(f, stream), "launch finalize kernel");
   }
 }
 
 void InferenceRunner::RunDevice(const float *deviceInputs, void *deviceResults, int64_t rows) {
   const int runs = gMeasureGpuKernelTime ? std::max(1, gNumberOfKernelRuns) : 1;
+  const Workspace ws = OwnWorkspace(rows);
   if (gMeasureGpuKernelTime) Check(hipEventRecord(m_evStart, m_stream), "hipEventRecord");
   for (int i = 0; i < runs; ++i) {
     if (ClassIdsAsInt8())
-      Launch(deviceInputs, rows, nullptr, static_cast<int8_t *>(deviceResults), nullptr, nullptr, nullptr);
+      Launch(deviceInputs, rows, nullptr, static_cast<int8_t *>(deviceResults), nullptr, nullptr, nullptr, m_stream, ws);
     else
-      Launch(deviceInputs, rows, static_cast<float *>(deviceResults), nullptr, nullptr, nullptr, nullptr);
+      Launch(deviceInputs, rows, static_cast<float *>(deviceResults), nullptr, nullptr, nullptr, nullptr, m_stream, ws);
   }
   if (gMeasureGpuKernelTime) Check(hipEventRecord(m_evStop, m_stream), "hipEventRecord");
   Check(hipStreamSynchronize(m_stream), "inference kernels");
@@ -268,20 +276,32 @@ void InferenceRunner::RunDevice(const float *deviceInputs, void *deviceResults, 
   }
 }
 
+void InferenceRunner::RunDeviceOnStream(const float *deviceInputs, void *deviceResults, int64_t rows, hipStream_t stream) {
+  if (rows < 0) throw Error("negative row count");
+  if (rows > 0 && (!deviceInputs || !deviceResults)) throw Error("null device buffer");
+  // Growing the runner's buffers waits for the runner's own stream only; an earlier call on another
+  // stream that still uses them must have finished before a call with more rows is made.
+  const Workspace ws = OwnWorkspace(rows);
+  if (ClassIdsAsInt8())
+    Launch(deviceInputs, rows, nullptr, static_cast<int8_t *>(deviceResults), nullptr, nullptr, nullptr, stream, ws);
+  else
+    Launch(deviceInputs, rows, static_cast<float *>(deviceResults), nullptr, nullptr, nullptr, nullptr, stream, ws);
+}
+
 void InferenceRunner::RunDeviceMulticlass(const float *deviceInputs, int64_t rows, int8_t *classIds, float *margins,
                                           float *probabilities) {
   if (m_forest.numClasses == 0) throw Error("model is not a multiclass classifier");
-  Launch(deviceInputs, rows, nullptr, classIds, margins, probabilities, nullptr);
+  Launch(deviceInputs, rows, nullptr, classIds, margins, probabilities, nullptr, m_stream, OwnWorkspace(rows));
   Check(hipStreamSynchronize(m_stream), "inference kernels");
 }
 
 void InferenceRunner::DumpLeafIds(const float *deviceInputs, int32_t *deviceLeafIds, int64_t rows) {
-  // results of the prediction itself are discarded into the staging buffers
-  EnsurePartial(rows);
+  // results of the prediction itself are discarded
+  const Workspace ws = OwnWorkspace(rows);
   float *scratch = nullptr;
   Check(hipMalloc(reinterpret_cast<void **>(&scratch), std::max<int64_t>(rows, 1) * sizeof(float)), "allocate scratch");
   try {
-    Launch(deviceInputs, rows, scratch, reinterpret_cast<int8_t *>(scratch), nullptr, nullptr, deviceLeafIds);
+    Launch(deviceInputs, rows, scratch, reinterpret_cast<int8_t *>(scratch), nullptr, nullptr, deviceLeafIds, m_stream, ws);
     Check(hipStreamSynchronize(m_stream), "leaf-id kernels");
   } catch (...) {
     (void)hipFree(scratch);
@@ -357,6 +377,7 @@ void InferenceRunner::RunHostChunk(const void *hostInputs, void *hostResults, in
       }
       if (!m_copier) m_copier.reset(new ParallelCopier((int)std::min(8u, std::max(1u, std::thread::hardware_concurrency()))));
     }
+    const Workspace ws = OwnWorkspace(perPiece); // the pieces run one after the other on the runner's stream
     int p = 0;
     for (int64_t first = 0; first < rows; first += perPiece, ++p) {
       const int64_t count = std::min(perPiece, rows - first);
@@ -371,9 +392,9 @@ void InferenceRunner::RunHostChunk(const void *hostInputs, void *hostResults, in
       Check(hipEventRecord(m_pieceReady[p], m_copyStream), "hipEventRecord");
       Check(hipStreamWaitEvent(m_stream, m_pieceReady[p], 0), "hipStreamWaitEvent");
       if (ClassIdsAsInt8())
-        Launch(dIn, count, nullptr, static_cast<int8_t *>(m_dStageOut) + first, nullptr, nullptr, nullptr);
+        Launch(dIn, count, nullptr, static_cast<int8_t *>(m_dStageOut) + first, nullptr, nullptr, nullptr, m_stream, ws);
       else
-        Launch(dIn, count, static_cast<float *>(m_dStageOut) + first, nullptr, nullptr, nullptr, nullptr);
+        Launch(dIn, count, static_cast<float *>(m_dStageOut) + first, nullptr, nullptr, nullptr, nullptr, m_stream, ws);
     }
     Check(hipStreamSynchronize(m_stream), "inference kernels");
   }
@@ -383,15 +404,14 @@ void InferenceRunner::RunHostChunk(const void *hostInputs, void *hostResults, in
 void InferenceRunner::TimeKernels(const float *deviceInputs, void *deviceResults, int64_t rows, int32_t runs,
                                   double *walkMs, double *finalizeMs, double *binMs) {
   runs = std::max(1, runs);
-  EnsurePartial(rows);
+  const Workspace ws = OwnWorkspace(rows);
   const bool finalize = NeedsFinalize();
   float ms = 0.f;
   if (binMs) *binMs = 0.0;
   const float *walkInputs = deviceInputs;
   if (m_model.plan.quantizedRows) {
-    EnsureRanks(rows);
     Check(hipEventRecord(m_evStart, m_stream), "hipEventRecord");
-    for (int i = 0; i < runs; ++i) walkInputs = PrepareRows(deviceInputs, rows);
+    for (int i = 0; i < runs; ++i) walkInputs = PrepareRows(deviceInputs, rows, ws.ranks, m_stream);
     Check(hipEventRecord(m_evStop, m_stream), "hipEventRecord");
     Check(hipStreamSynchronize(m_stream), "rank-quantisation kernel");
     Check(hipEventElapsedTime(&ms, m_evStart, m_evStop), "hipEventElapsedTime");
@@ -399,9 +419,9 @@ void InferenceRunner::TimeKernels(const float *deviceInputs, void *deviceResults
   }
   WalkParams p = MakeWalkParams(walkInputs, rows);
   p.out = finalize ? nullptr : static_cast<float *>(deviceResults);
-  p.partial = finalize ? m_dPartial : nullptr;
+  p.partial = finalize ? ws.partial : nullptr;
   Check(hipEventRecord(m_evStart, m_stream), "hipEventRecord");
-  for (int i = 0; i < runs; ++i) Check(LaunchWalk(p), "launch walk kernel");
+  for (int i = 0; i < runs; ++i) Check(LaunchWalk(p, m_stream), "launch walk kernel");
   Check(hipEventRecord(m_evStop, m_stream), "hipEventRecord");
   Check(hipStreamSynchronize(m_stream), "walk kernel");
   Check(hipEventElapsedTime(&ms, m_evStart, m_evStop), "hipEventElapsedTime");
@@ -409,7 +429,7 @@ void InferenceRunner::TimeKernels(const float *deviceInputs, void *deviceResults
   if (finalizeMs) *finalizeMs = 0.0;
   if (finalize) {
     FinalizeParams f;
-    f.partial = m_dPartial;
+    f.partial = ws.partial;
     f.rows = rows;
     f.numClasses = m_forest.numClasses;
     f.treeSlices = m_model.PartialCount();

@@ -41,6 +41,9 @@ public:
   void RunHost(const void *hostInputs, void *hostResults, int64_t rows);
   // Device-resident rows; `out` holds ReturnTypeBytes() per row.
   void RunDevice(const float *deviceInputs, void *deviceResults, int64_t rows);
+  // The same kernels enqueued on the caller's stream; returns without waiting for them.  Work the caller
+  // queued on that stream before the call is seen by the kernels, work queued after it sees their results.
+  void RunDeviceOnStream(const float *deviceInputs, void *deviceResults, int64_t rows, hipStream_t stream);
   // Multiclass extras: any of the outputs may be null.
   void RunDeviceMulticlass(const float *deviceInputs, int64_t rows, int8_t *classIds, float *margins,
                            float *probabilities);
@@ -80,13 +83,22 @@ private:
   void EnsurePartial(int64_t rows);
   void EnsureStaging(int64_t rows);
   void EnsureRanks(int64_t rows);
+  // Device memory the kernels of one call use beyond inputs and outputs.
+  struct Workspace {
+    double *partial = nullptr; // [PartialCount()][rows][max(1, classes)] when NeedsFinalize()
+    uint8_t *ranks = nullptr;  // rank-quantised rows when the plan uses them
+  };
+  // Allocating callers: grows the runner's own buffers to hold `rows` rows.
+  Workspace OwnWorkspace(int64_t rows);
+  size_t PartialBytes(int64_t rows) const;
+  size_t RanksBytes(int64_t rows) const;
   // Rank-quantised plans: runs the binning kernel and returns the buffer the walk kernel reads.
-  const float *PrepareRows(const float *deviceInputs, int64_t rows);
+  const float *PrepareRows(const float *deviceInputs, int64_t rows, uint8_t *ranks, hipStream_t stream);
   bool NeedsFinalize() const { return m_model.plan.treeSlices > 1 || m_forest.numClasses > 0; }
   WalkParams MakeWalkParams(const float *deviceInputs, int64_t rows) const;
-  hipError_t LaunchWalk(const WalkParams &p) const;
+  hipError_t LaunchWalk(const WalkParams &p, hipStream_t stream) const;
   void Launch(const float *deviceInputs, int64_t rows, float *out, int8_t *classOut, float *margins,
-              float *probabilities, int32_t *leafIds);
+              float *probabilities, int32_t *leafIds, hipStream_t stream, const Workspace &ws);
 
   Forest m_forest;
   CompilerOptions m_options;

@@ -316,6 +316,10 @@ int32_t tbmi_run_device(intptr_t h, const float *in, void *out, int64_t rows) {
   return Guard([&] { Runner(h)->RunDevice(in, out, rows); return 0; }, -1);
 }
 
+int32_t tbmi_run_device_async(intptr_t h, const float *in, void *out, int64_t rows, void *stream) {
+  return Guard([&] { Runner(h)->RunDeviceOnStream(in, out, rows, static_cast<hipStream_t>(stream)); return 0; }, -1);
+}
+
 int32_t tbmi_run_host(intptr_t h, const void *in, void *out, int64_t rows) {
   return Guard(
       [&] {

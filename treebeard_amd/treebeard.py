@@ -287,6 +287,11 @@ class TreebeardInferenceRunner:
         self._rc(_lib().tbmi_run_device(self.inferenceRunner, device_inputs_ptr, device_results_ptr, rows),
                  "tbmi_run_device")
 
+    def run_device_async(self, device_inputs_ptr, device_results_ptr, rows, stream=None):
+        """Enqueues the kernels on `stream` (a hipStream_t address, None = the default stream) and returns."""
+        self._rc(_lib().tbmi_run_device_async(self.inferenceRunner, device_inputs_ptr, device_results_ptr, rows,
+                                              stream), "tbmi_run_device_async")
+
     def run_device_multiclass(self, device_inputs_ptr, rows, class_ids_ptr=None, margins_ptr=None, probs_ptr=None):
         self._rc(_lib().tbmi_run_device_multiclass(self.inferenceRunner, device_inputs_ptr, rows, class_ids_ptr,
                                                    margins_ptr, probs_ptr), "tbmi_run_device_multiclass")
