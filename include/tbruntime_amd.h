@@ -128,6 +128,17 @@ TBAMD_EXPORT int32_t tbmi_run_device(intptr_t runner, const float *deviceInputs,
  * call is made no earlier call on another stream may still be running. */
 TBAMD_EXPORT int32_t tbmi_run_device_async(intptr_t runner, const float *deviceInputs, void *deviceResults,
                                            int64_t rows, void *stream);
+/* No counterpart in the reference.  For callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): tbmi_run_device_async with the kernels'
+ * scratch memory (partial sums of classifiers and of plans that split the trees over several blocks, the
+ * rank-quantised rows of wide models) taken from one fixed device array of tbmi_noalloc_scratch_bytes()
+ * bytes (32 MiB) that the library holds on every GPU it runs on.  It allocates, frees and synchronises
+ * nothing.  A call whose plan needs more scratch memory than that for `rows` rows fails with a message
+ * naming both sizes (pass fewer rows per call).  All calls on one GPU share the array: calls that overlap
+ * in time on one GPU, from any runner or stream, race on it. */
+TBAMD_EXPORT int32_t tbmi_run_device_noalloc(intptr_t runner, const float *deviceInputs, void *deviceResults,
+                                             int64_t rows, void *stream);
+TBAMD_EXPORT int64_t tbmi_noalloc_scratch_bytes(void);
 /* Host buffers like RunInference, but any number of rows (the reference fixes the batch at compile time,
  * src/runtime/runtime.cpp:58-67): batch-sized windows, copies overlapped with the kernels. */
 TBAMD_EXPORT int32_t tbmi_run_host(intptr_t runner, const void *hostInputs, void *hostResults, int64_t rows);

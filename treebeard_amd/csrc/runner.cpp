@@ -1,6 +1,7 @@
 #include "runner.h"
 
 #include <algorithm>
+#include <mutex>
 #include <sstream>
 
 namespace tbamd {
@@ -12,6 +13,39 @@ namespace {
 
 void Check(hipError_t e, const char *what) {
   if (e != hipSuccess) throw Error(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+// Scratch memory of the entry point that allocates nothing (RunDeviceNoAlloc): partial sums and
+// rank-quantised rows of one call.  Every GPU the library runs on holds its own copy of the array
+// until the process ends.  In host code the array's name is only a handle for the runtime: the
+// address kernels can use is looked up once per device and kept in gScratchAddress.
+constexpr size_t kNoAllocScratchBytes = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+constexpr int kMaxDevices = 64;
+unsigned char *gScratchAddress[kMaxDevices] = {};
+std::mutex gScratchMutex;
+
+// Device address of `scratch` on the current device (looked up on first use, then cached).
+unsigned char *ScratchOfCurrentDevice() {
+  int device = -1;
+  Check(hipGetDevice(&device), "hipGetDevice");
+  if (device < 0 || device >= kMaxDevices) throw Error("device index out of range for the fixed scratch array");
+  std::lock_guard<std::mutex> lock(gScratchMutex);
+  if (!gScratchAddress[device]) {
+    void *address = nullptr;
+    Check(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)), "hipGetSymbolAddress");
+    if (!address) throw Error("hipGetSymbolAddress returned no address for the fixed scratch array");
+    gScratchAddress[device] = static_cast<unsigned char *>(address);
+  }
+  return gScratchAddress[device];
+}
+
+template <typename T> T *Upload(const std::vector<T> &host, const char *what) {
+  T *ptr = nullptr;
+  const size_t bytes = std::max<size_t>(host.size(), 1) * sizeof(T);
+  Check(hipMalloc(reinterpret_cast<void **>(&ptr), bytes), what);
+  if (!host.empty()) Check(hipMemcpy(ptr, host.data(), host.size() * sizeof(T), hipMemcpyHostToDevice), what);
+  return ptr;
 }
 
 } // namespace
@@ -59,6 +93,7 @@ void InferenceRunner::InitDevice() {
   Check(hipGetDeviceProperties(&prop, 0), "hipGetDeviceProperties");
   m_limits.computeUnits = prop.multiProcessorCount;
   m_limits.ldsBytesPerBlock = (int32_t)std::min<size_t>(prop.sharedMemPerBlock, 160 * 1024);
+  (void)ScratchOfCurrentDevice(); // set-up: the no-allocation entry point finds its array's address ready
   Check(hipStreamCreateWithFlags(&m_stream, hipStreamNonBlocking), "hipStreamCreate");
   Check(hipEventCreate(&m_evStart), "hipEventCreate");
   Check(hipEventCreate(&m_evStop), "hipEventCreate");
@@ -282,6 +317,30 @@ void InferenceRunner::RunDeviceOnStream(const float *deviceInputs, void *deviceR
   // Growing the runner's buffers waits for the runner's own stream only; an earlier call on another
   // stream that still uses them must have finished before a call with more rows is made.
   const Workspace ws = OwnWorkspace(rows);
+  if (ClassIdsAsInt8())
+    Launch(deviceInputs, rows, nullptr, static_cast<int8_t *>(deviceResults), nullptr, nullptr, nullptr, stream, ws);
+  else
+    Launch(deviceInputs, rows, static_cast<float *>(deviceResults), nullptr, nullptr, nullptr, nullptr, stream, ws);
+}
+
+size_t InferenceRunner::NoAllocScratchBytes() { return kNoAllocScratchBytes; }
+
+void InferenceRunner::RunDeviceNoAlloc(const float *deviceInputs, void *deviceResults, int64_t rows, hipStream_t stream) {
+  if (rows < 0) throw Error("negative row count");
+  if (rows == 0) return;
+  if (!deviceInputs || !deviceResults) throw Error("null device buffer");
+  const size_t partialBytes = (PartialBytes(rows) + 255) & ~(size_t)255;
+  const size_t ranksBytes = RanksBytes(rows);
+  if (partialBytes + ranksBytes > kNoAllocScratchBytes)
+    throw Error("this launch plan needs " + std::to_string(partialBytes + ranksBytes) + " bytes of scratch memory for " +
+                std::to_string(rows) + " rows; the fixed array of the no-allocation entry point holds " +
+                std::to_string(kNoAllocScratchBytes) + ": pass fewer rows per call or use tbmi_run_device_async");
+  unsigned char *base = ScratchOfCurrentDevice();
+  Workspace ws;
+  ws.partial = reinterpret_cast<double *>(base);
+  ws.ranks = base + partialBytes;
+  // Every partial sum the finalize kernel reads and every rank the walk reads is written earlier in
+  // this same call, so nothing has to be cleared between calls.
   if (ClassIdsAsInt8())
     Launch(deviceInputs, rows, nullptr, static_cast<int8_t *>(deviceResults), nullptr, nullptr, nullptr, stream, ws);
   else

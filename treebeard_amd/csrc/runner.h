@@ -44,6 +44,12 @@ public:
   // The same kernels enqueued on the caller's stream; returns without waiting for them.  Work the caller
   // queued on that stream before the call is seen by the kernels, work queued after it sees their results.
   void RunDeviceOnStream(const float *deviceInputs, void *deviceResults, int64_t rows, hipStream_t stream);
+  // As RunDeviceOnStream, but the partial sums and rank-quantised rows go into the library's fixed
+  // device array instead of allocated buffers: no allocation, no free, no synchronisation.  Throws when
+  // the plan needs more than NoAllocScratchBytes() for `rows` rows.
+  void RunDeviceNoAlloc(const float *deviceInputs, void *deviceResults, int64_t rows, hipStream_t stream);
+  // Bytes of the fixed device array the no-allocation entry point may use.
+  static size_t NoAllocScratchBytes();
   // Multiclass extras: any of the outputs may be null.
   void RunDeviceMulticlass(const float *deviceInputs, int64_t rows, int8_t *classIds, float *margins,
                            float *probabilities);

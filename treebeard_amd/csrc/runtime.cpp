@@ -320,6 +320,12 @@ int32_t tbmi_run_device_async(intptr_t h, const float *in, void *out, int64_t ro
   return Guard([&] { Runner(h)->RunDeviceOnStream(in, out, rows, static_cast<hipStream_t>(stream)); return 0; }, -1);
 }
 
+int32_t tbmi_run_device_noalloc(intptr_t h, const float *in, void *out, int64_t rows, void *stream) {
+  return Guard([&] { Runner(h)->RunDeviceNoAlloc(in, out, rows, static_cast<hipStream_t>(stream)); return 0; }, -1);
+}
+
+int64_t tbmi_noalloc_scratch_bytes(void) { return (int64_t)InferenceRunner::NoAllocScratchBytes(); }
+
 int32_t tbmi_run_host(intptr_t h, const void *in, void *out, int64_t rows) {
   return Guard(
       [&] {

@@ -54,6 +54,8 @@ SIGNATURES = {
     "tbmi_device_count": (c_i32, []),
     "tbmi_run_device": (c_i32, [c_ip, c_vp, c_vp, c_i64]),
     "tbmi_run_device_async": (c_i32, [c_ip, c_vp, c_vp, c_i64, c_vp]),
+    "tbmi_run_device_noalloc": (c_i32, [c_ip, c_vp, c_vp, c_i64, c_vp]),
+    "tbmi_noalloc_scratch_bytes": (c_i64, []),
     "tbmi_run_device_multiclass": (c_i32, [c_ip, c_vp, c_i64, c_vp, c_vp, c_vp]),
     "tbmi_dump_leaf_ids": (c_i32, [c_ip, c_vp, c_vp, c_i64]),
     "tbmi_time_kernels": (c_i32, [c_ip, c_vp, c_vp, c_i64, c_i32, ctypes.POINTER(ctypes.c_double),

@@ -292,6 +292,11 @@ class TreebeardInferenceRunner:
         self._rc(_lib().tbmi_run_device_async(self.inferenceRunner, device_inputs_ptr, device_results_ptr, rows,
                                               stream), "tbmi_run_device_async")
 
+    def run_device_noalloc(self, device_inputs_ptr, device_results_ptr, rows, stream=None):
+        """run_device_async without any allocation: scratch memory comes from the library's fixed device array."""
+        self._rc(_lib().tbmi_run_device_noalloc(self.inferenceRunner, device_inputs_ptr, device_results_ptr, rows,
+                                                stream), "tbmi_run_device_noalloc")
+
     def run_device_multiclass(self, device_inputs_ptr, rows, class_ids_ptr=None, margins_ptr=None, probs_ptr=None):
         self._rc(_lib().tbmi_run_device_multiclass(self.inferenceRunner, device_inputs_ptr, rows, class_ids_ptr,
                                                    margins_ptr, probs_ptr), "tbmi_run_device_multiclass")
