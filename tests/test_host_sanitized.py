@@ -1,6 +1,14 @@
-"""The host side of the library (loaders, packer, tuner, compiled-model file, the pinned-staging copier)
-compiled with AddressSanitizer + UndefinedBehaviorSanitizer and driven over the five configurations with
-every launch-plan shape the GPU tests pin.  No GPU and no HIP runtime involved."""
+"""The host side of the library compiled with sanitizers, no GPU and no HIP runtime involved.
+
+test_host_code_under_sanitizers: loaders, packer, tuner, compiled-model file and the pinned-staging copier
+under AddressSanitizer + UndefinedBehaviorSanitizer over the five configurations with every launch-plan shape
+the GPU tests pin.
+
+test_runner_under_*: the runner and the whole C ABI (runner.cpp, runtime.cpp) linked against a host-only
+stand-in for the HIP runtime whose "kernels" interpret the packed model on the CPU (tests/native/
+hip_host_shim.cpp), driven through host and device entry points of many sizes, plan changes, the plan search
+and the compiled-model file: every buffer the runner sizes and every copy it makes is seen by ASan/UBSan, the
+copier threads by ThreadSanitizer."""
 import os
 import shutil
 import subprocess
@@ -29,3 +37,53 @@ def test_host_code_under_sanitizers(tmp_path, synth_model):
     run = subprocess.run([exe] + models, capture_output=True, text=True, env=env, timeout=900)
     assert run.returncode == 0, (run.stdout + run.stderr)[-4000:]
     assert "ok" in run.stdout
+
+
+RUNNER_SOURCES = HOST_SOURCES + ["onnx_loader.cpp", "runner.cpp", "runtime.cpp"]
+
+
+def _build_runner_driver(tmp_path, sanitize):
+    exe = str(tmp_path / ("sanitize_runner_" + sanitize.split(",")[0]))
+    cmd = ["g++", "-std=c++17", "-O1", "-g", "-fsanitize=" + sanitize, "-fno-omit-frame-pointer",
+           "-D__HIP_PLATFORM_AMD__", "-D__align__(x)=__attribute__((aligned(x)))", "-DHIP_SYMBOL(x)=x",
+           "-I", "/opt/rocm/include", "-I", CSRC,
+           os.path.join(HERE, "native", "sanitize_runner.cpp"), os.path.join(HERE, "native", "hip_host_shim.cpp")]
+    if "undefined" in sanitize:
+        cmd.append("-fno-sanitize-recover=undefined")
+    cmd += [os.path.join(CSRC, s) for s in RUNNER_SOURCES] + ["-lpthread", "-o", exe]
+    built = subprocess.run(cmd, capture_output=True, text=True)
+    if built.returncode != 0 and ("sanitize" in built.stderr or "hip/hip_runtime" in built.stderr):
+        pytest.skip("this g++ has no sanitizer runtime, or the HIP headers are missing")
+    assert built.returncode == 0, built.stderr[-3000:]
+    return exe
+
+
+def _wide_model(tmp_path):
+    """40 trees over 600 features: 8300 rows are 20 MB of input, enough for the host entry point to send them
+    in pieces through its pinned buffers, and cheap to walk on the CPU."""
+    import numpy as np
+    rng = np.random.Generator(np.random.PCG64(5))
+    trees = [synth._grow_tree(rng, 6, lambda d, s: 0.9, lambda: (rng.integers(0, 600), rng.standard_normal()),
+                              lambda: rng.normal(0.0, 0.1)) for _ in range(40)]
+    path = str(tmp_path / "wide600.json")
+    synth.write_xgboost_json(path, trees, 600)
+    return path
+
+
+@pytest.mark.skipif(shutil.which("g++") is None, reason="needs g++")
+def test_runner_under_address_sanitizer(tmp_path, synth_model):
+    exe = _build_runner_driver(tmp_path, "address,undefined")
+    args = [_wide_model(tmp_path), "8300", synth_model(4), "300", synth_model(3), "1500", synth_model(1), "20000"]
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", TMPDIR=str(tmp_path))
+    run = subprocess.run([exe] + args, capture_output=True, text=True, env=env, timeout=900)
+    assert run.returncode == 0, (run.stdout + run.stderr)[-4000:]
+    assert run.stdout.strip().endswith("ok")
+
+
+@pytest.mark.skipif(shutil.which("g++") is None, reason="needs g++")
+def test_runner_under_thread_sanitizer(tmp_path, synth_model):
+    exe = _build_runner_driver(tmp_path, "thread")
+    env = dict(os.environ, SANITIZE_QUICK="1", TMPDIR=str(tmp_path))
+    run = subprocess.run([exe, _wide_model(tmp_path), "8300"], capture_output=True, text=True, env=env, timeout=900)
+    assert run.returncode == 0, (run.stdout + run.stderr)[-4000:]
+    assert run.stdout.strip().endswith("ok")
