@@ -231,6 +231,93 @@ hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, int tileMode, 
   return WalkLds(p, interleave, stride, tileMode == 2);
 }
 
+namespace {
+
+// One tile step of the tiled layout (device_model.h): returns the byte address of the child tile.
+uint32_t TileStepHost(const unsigned char *group, uint32_t groupBytes, uint32_t addr, int T, const float *row, int F,
+                      uint32_t stride) {
+  const uint32_t bytes = TileBytes(T);
+  if (addr % 8 != 0 || addr + bytes > groupBytes) std::abort(); // tile outside the group
+  const unsigned char *tile = group + addr;
+  float thr[kMaxTileSize];
+  uint16_t off[kMaxTileSize], childBase;
+  std::memcpy(thr, tile, (size_t)T * 4);
+  std::memcpy(off, tile + T * 4, (size_t)T * 2);
+  std::memcpy(&childBase, tile + T * 6, 2);
+  uint64_t select = 0;
+  if (T == 4) {
+    uint16_t low;
+    uint32_t high;
+    std::memcpy(&low, tile + 26, 2);
+    std::memcpy(&high, tile + 28, 4);
+    select = (uint64_t)low | ((uint64_t)high << 16);
+  } else {
+    uint16_t s16;
+    std::memcpy(&s16, tile + T * 6 + 2, 2);
+    select = s16;
+  }
+  uint32_t outcome = 0;
+  for (int i = 0; i < T; ++i) {
+    if (off[i] % stride != 0 || (int)(off[i] / stride) > F) std::abort();
+    const int f = (int)(off[i] / stride);
+    const float x = f == F ? -INFINITY : row[f];
+    outcome |= (x < thr[i] ? 1u : 0u) << i;
+  }
+  const uint32_t width = TileSelectBits(T);
+  const uint32_t child = (uint32_t)(select >> (outcome * width)) & ((1u << width) - 1u);
+  return childBase + child * bytes;
+}
+
+} // namespace
+
+hipError_t LaunchWalkRowsTiled(const WalkParams &p, int tileSize, int interleave, size_t ldsBytes, hipStream_t) {
+  if (p.s.rows <= 0) return hipSuccess;
+  const int RB = p.s.rowsPerBlock, TT = p.s.treeThreads, T = tileSize, K = interleave;
+  if (ldsBytes > 160 * 1024 || RB < 64 || (RB & (RB - 1)) || TT < 1 || RB * TT > 1024) return hipErrorInvalidValue;
+  if ((int64_t)(p.s.numFeatures + 1) * RB * 4 > 0x10000) return hipErrorInvalidValue;
+  if (p.s.treeSlices < 1 || p.s.treeSlices > 65535) return hipErrorInvalidValue;
+  if ((int)((p.s.groupRegionBytes / 16 + RB * TT - 1) / (RB * TT)) > 16) return hipErrorInvalidValue;
+  if (T < 2 || T > 4 || (K != 1 && K != 2 && K != 4)) return hipErrorInvalidValue;
+  if (p.s.treeSlices > 1 && !p.partial) std::abort();
+  const DeviceNode *nodes = reinterpret_cast<const DeviceNode *>(p.nodes16);
+  const int F = p.s.numFeatures;
+  const int Cn = p.s.numClasses > 0 ? p.s.numClasses : 1;
+  std::vector<double> sums((size_t)Cn);
+  for (int slice = 0; slice < p.s.treeSlices; ++slice) {
+    const int gBegin = (int)(((int64_t)p.s.numGroups * slice) / p.s.treeSlices);
+    const int gEnd = (int)(((int64_t)p.s.numGroups * (slice + 1)) / p.s.treeSlices);
+    for (int64_t row = 0; row < p.s.rows; ++row) {
+      std::fill(sums.begin(), sums.end(), 0.0);
+      for (int g = gBegin; g < gEnd; ++g) {
+        const DeviceGroup grp = p.groups[g];
+        const unsigned char *group = reinterpret_cast<const unsigned char *>(nodes + grp.nodeBegin);
+        for (uint32_t b = 0; b < grp.bundleCount; ++b) {
+          const DeviceBundle bd = p.bundles[grp.bundleBegin + b];
+          if (bd.peelDepth > bd.depth) std::abort();
+          for (int k = 0; k < K; ++k) {
+            uint32_t addr = bd.root[k];
+            // the kernel stops early only when no lane moves any more, which leaves every lane where `depth`
+            // steps would: the full walk is the specification
+            for (uint32_t d = 0; d < bd.depth; ++d)
+              addr = TileStepHost(group, grp.nodeCount * kNodeBytes, addr, T, p.x + row * F, F, (uint32_t)RB * 4u);
+            const uint32_t settled = TileStepHost(group, grp.nodeCount * kNodeBytes, addr, T, p.x + row * F, F, (uint32_t)RB * 4u);
+            if (settled != addr) std::abort(); // `depth` steps must end on a leaf tile
+            float value;
+            std::memcpy(&value, group + addr, 4);
+            sums[p.s.numClasses > 0 ? bd.classId : 0] += (double)value;
+            if (p.leafIds) {
+              const int tree = p.slotTree[bd.firstSlot + k];
+              if (tree >= 0) p.leafIds[row * p.s.numTrees + tree] = p.nodeOrigin[grp.nodeBegin + addr / kNodeBytes];
+            }
+          }
+        }
+      }
+      StoreRow(p, row, slice, sums.data());
+    }
+  }
+  return hipSuccess;
+}
+
 hipError_t LaunchWalkTreeParallel(const WalkParams &p, int interleave, size_t ldsBytes, hipStream_t) {
   if (p.s.rows <= 0) return hipSuccess;
   if (ldsBytes > 160 * 1024 || p.s.rowsPerBlock < 1 || p.s.treeLanes < 1) return hipErrorInvalidValue;

@@ -105,16 +105,48 @@ void Compare(const Case &c, const float *got, int64_t first, int64_t rows, const
   EXPECT(bad == 0, "%s: %lld of %lld rows differ (%s)", what, (long long)bad, (long long)rows, c.path.c_str());
 }
 
-intptr_t MakeRunner(const Case &c, int32_t batch, bool int8Classes) {
+// Leaf hit counts of the case's own rows in the reference's profile format (first line `numTrees, numRows`,
+// then per tree `hitCount, depth` for every leaf in node order).
+std::string WriteProfile(const Case &c, const std::string &path) {
+  const int64_t F = c.forest.numFeatures;
+  const size_t T = c.forest.trees.size();
+  std::vector<std::vector<int64_t>> hits(T);
+  for (size_t t = 0; t < T; ++t) hits[t].assign(c.forest.trees[t].value.size(), 0);
+  std::vector<int32_t> ids(T);
+  for (int64_t r = 0; r < c.rows; ++r) {
+    Predict(c.forest, c.x.data() + r * F, ids.data());
+    for (size_t t = 0; t < T; ++t) ++hits[t][ids[t]];
+  }
+  FILE *out = std::fopen(path.c_str(), "w");
+  std::fprintf(out, "%zu, %lld\n", T, (long long)c.rows);
+  for (size_t t = 0; t < T; ++t) {
+    const HostTree &tree = c.forest.trees[t];
+    bool first = true;
+    for (size_t n = 0; n < tree.value.size(); ++n) {
+      if (tree.left[n] != -1) continue;
+      std::fprintf(out, "%s%lld, 0", first ? "" : ", ", (long long)hits[t][n]);
+      first = false;
+    }
+    std::fprintf(out, "\n");
+  }
+  std::fclose(out);
+  return path;
+}
+
+intptr_t MakeRunner(const Case &c, int32_t batch, bool int8Classes, int32_t tileSize = 1, int32_t tilingType = 0,
+                    const char *profile = "") {
   const intptr_t options = CreateCompilerOptions();
   Set_batchSize(options, batch);
+  Set_tileSize(options, tileSize);
+  Set_tilingType(options, tilingType);
+  Set_statsProfileCSVPath(options, profile);
   if (int8Classes) {
     Set_returnTypeWidth(options, 8);
     Set_returnTypeFloatType(options, 0);
   }
   const intptr_t runner = CreateInferenceRunner(c.path.c_str(), "", options);
   DeleteCompilerOptions(options);
-  EXPECT(runner != 0, "CreateInferenceRunner");
+  EXPECT(runner != 0 || tileSize > 1, "CreateInferenceRunner");
   return runner;
 }
 
@@ -160,12 +192,26 @@ void HostEntryPoints(const Case &c) {
   }
 }
 
-void DeviceEntryPoints(const Case &c, int64_t rows) {
+void DeviceEntryPoints(const Case &c, int64_t rows, int32_t tileSize = 1, int32_t tilingType = 0, const char *profile = "",
+                       bool peel = false) {
   const int64_t F = c.forest.numFeatures;
   const int32_t T = (int32_t)c.forest.trees.size();
   const bool multiclass = c.forest.numClasses > 0;
-  const intptr_t runner = MakeRunner(c, (int32_t)rows, multiclass);
-  if (!runner) return;
+  SetPeeledCodeGenForProbabilityBasedTiling(peel ? 1 : 0);
+  const intptr_t runner = MakeRunner(c, (int32_t)rows, multiclass, tileSize, tilingType, profile);
+  SetPeeledCodeGenForProbabilityBasedTiling(0);
+  if (!runner) {
+    // tiled walks are refused where the row tile cannot hold byte offsets (very wide rows), never silently dropped
+    EXPECT(tileSize > 1 && std::strstr(tbmi_last_error(), "tile size"), "runner with tile size %d", tileSize);
+    return;
+  }
+  {
+    char plan[1024];
+    tbmi_describe_plan(runner, plan, sizeof(plan));
+    char want[64];
+    std::snprintf(want, sizeof(want), " tileSize=%d ", tileSize);
+    EXPECT(std::strstr(plan, want) != nullptr, "plan does not carry the tile size: %s", plan);
+  }
   float *dx = nullptr;
   void *dout = nullptr;
   int32_t *dids = nullptr;
@@ -202,7 +248,29 @@ void DeviceEntryPoints(const Case &c, int64_t rows) {
     EXPECT(tbmi_describe_plan(runner, big, sizeof(big)) > 0, "describe");
   };
   runAll("default plan");
-  if (Quick()) {
+  if (tileSize > 1) { // block shapes of the tiled walk, the plan search, save and reload
+    const int tiledPlans[][5] = {{64, 1, 1, 16384, 1}, {128, 8, 2, 32768, 3}, {256, 4, 4, 40960, 2}, {64, 16, 2, 24576, 5}};
+    for (auto &p : tiledPlans)
+      if (tbmi_set_plan(runner, p[0], p[1], p[2], p[3], p[4]) == 0) runAll("tiled plan");
+    EXPECT(tbmi_set_tree_parallel_plan(runner, 4, 64, 1, 0, 1) == -1, "tree-parallel plan must refuse tiles");
+    double best = 0;
+    EXPECT(tbmi_autotune(runner, dx, rows, &best) == 0, "tbmi_autotune (tiled)");
+    runAll("tiled, after the plan search");
+    const std::string file = std::string(std::getenv("TMPDIR") ? std::getenv("TMPDIR") : "/tmp") + "/sanitize_tiled.tbamd";
+    EXPECT(tbmi_save_compiled_model(runner, file.c_str()) == 0, "tbmi_save_compiled_model (tiled)");
+    const intptr_t again = tbmi_load_compiled_model(file.c_str(), 0);
+    EXPECT(again != 0, "tbmi_load_compiled_model (tiled)");
+    if (again) {
+      char a[1024], b[1024];
+      tbmi_describe_plan(runner, a, sizeof(a));
+      tbmi_describe_plan(again, b, sizeof(b));
+      EXPECT(std::strcmp(a, b) == 0, "reloaded tiled plan differs: %s / %s", a, b);
+      EXPECT(tbmi_run_device(again, dx, dout, rows) == 0, "reloaded tiled runner");
+      check("reloaded tiled runner");
+      DeleteInferenceRunner(again);
+    }
+  }
+  if (Quick() || tileSize > 1) {
     DeleteInferenceRunner(runner);
     (void)hipFree(dx);
     (void)hipFree(dout);
@@ -270,6 +338,22 @@ int main(int argc, char **argv) {
     for (int64_t r = 0; r < c.rows; ++r) c.expected[r] = Predict(c.forest, c.x.data() + r * F, nullptr);
     HostEntryPoints(c);
     DeviceEntryPoints(c, std::min<int64_t>(c.rows, 203));
+    if (!Quick()) {
+      const std::string profile =
+          WriteProfile(c, std::string(std::getenv("TMPDIR") ? std::getenv("TMPDIR") : "/tmp") + "/sanitize_profile.csv");
+      for (int32_t tileSize : {2, 3, 4}) {
+        DeviceEntryPoints(c, std::min<int64_t>(c.rows, 203), tileSize);
+        DeviceEntryPoints(c, std::min<int64_t>(c.rows, 203), tileSize, 1, profile.c_str(), true);
+        DeviceEntryPoints(c, std::min<int64_t>(c.rows, 203), tileSize, 2, profile.c_str(), false);
+      }
+      DeviceEntryPoints(c, std::min<int64_t>(c.rows, 203), 1, 1, profile.c_str(), true); // scalar nodes, peeled walks
+      const intptr_t options = CreateCompilerOptions();
+      Set_batchSize(options, 64);
+      Set_tileSize(options, 8);
+      EXPECT(CreateInferenceRunner(c.path.c_str(), "", options) == 0 && std::strstr(tbmi_last_error(), "tile size 8"),
+             "tile size 8 must be refused");
+      DeleteCompilerOptions(options);
+    }
     std::printf("%s: %lld rows done, %d failures so far\n", argv[a], (long long)c.rows, gFailures);
     std::fflush(stdout);
   }

@@ -755,3 +755,117 @@ def test_async_entry_point_orders_itself_on_the_callers_stream(synth_model, k, r
     pred, _ = cpu_oracle.predict(forest, x)
     if forest.num_classes == 0:
         np.testing.assert_allclose(expected, pred, rtol=RTOL_SUM, atol=ATOL_PROB)
+
+
+# --------------------------------------------------------------------------
+# tiled walks (CompilerOptions tile size 2, 3, 4) and probability-based tiling
+# --------------------------------------------------------------------------
+def make_tiled_runner(path, batch, tile_size, tiling_type=0, profile="", peel=False, multiclass=False):
+    options = treebeard.CompilerOptions(batch, tile_size)
+    options.SetTilingType(tiling_type)
+    if profile:
+        options.SetStatsProfileCSVPath(str(profile))
+    if multiclass:
+        options.SetReturnTypeWidth(8)
+        options.SetReturnTypeIsFloatType(False)
+    treebeard.SetPeeledCodeGenForProbabilityBasedTiling(peel)
+    try:
+        return treebeard.TreebeardInferenceRunner.FromModelFile(str(path), "", options)
+    finally:
+        treebeard.SetPeeledCodeGenForProbabilityBasedTiling(False)
+
+
+def write_profile(path, forest, ids):
+    """Leaf hit counts of a batch in the reference's profile format (src/utils/StatsUtils.cpp:10-52)."""
+    lines = ["%d, %d" % (forest.num_trees, ids.shape[0])]
+    for t in range(forest.num_trees):
+        _, _, left, _ = forest.tree(t)
+        counts = np.bincount(ids[:, t], minlength=len(left))
+        lines.append(", ".join("%d, 0" % counts[leaf] for leaf in np.nonzero(left == -1)[0]))
+    with open(path, "w") as fh:
+        fh.write("\n".join(lines) + "\n")
+    return str(path)
+
+
+@pytest.mark.parametrize("tile_size", [2, 3, 4])
+@pytest.mark.parametrize("k,rows", [(1, 1024), (2, 4096), (3, 4096), (5, 2048)])
+def test_tiled_walk_selects_the_scalar_walks_leaves(synth_model, k, rows, tile_size):
+    """Set_tileSize > 1 runs the tiled kernel; its leaves are those of the scalar oracle and of the tiled CPU walk."""
+    forest = model_io.load_xgboost_json(synth_model(k))
+    x = synth.CONFIGS[k].batch_rows(rows, seed_offset=4)
+    runner = make_tiled_runner(synth_model(k), rows, tile_size, multiclass=k == 3)
+    assert " tileSize=%d " % tile_size in runner.describe_plan()
+    ids = gpu_leaf_ids(runner, x)
+    np.testing.assert_array_equal(ids, cpu_oracle.leaf_ids(forest, x))
+    np.testing.assert_array_equal(ids, cpu_oracle.TiledForest(forest, tile_size).leaf_ids(x))
+    check_against_oracle(runner, forest, x)
+
+
+@pytest.mark.parametrize("tile_size", [2, 4])
+def test_tiled_walk_on_the_reference_fixtures(plain_file, tile_size):
+    for name in BENCHMARK_XGB:
+        path = plain_file(benchmark_model(name))
+        data = np.loadtxt(benchmark_csv(name), delimiter=",", dtype=np.float64)
+        x, expected = data[:, :-1].astype(np.float32), data[:, -1]
+        forest = model_io.load_xgboost_json(path)
+        runner = make_tiled_runner(path, x.shape[0], tile_size)
+        np.testing.assert_array_equal(gpu_leaf_ids(runner, x), cpu_oracle.leaf_ids(forest, x))
+        np.testing.assert_allclose(gpu_predict(runner, x), expected, rtol=RTOL_SUM, atol=ATOL_PROB)
+    for path in random_models()[::4]:
+        forest = model_io.load_xgboost_json(path)
+        x = np.random.default_rng(tile_size).random((777, forest.num_features), dtype=np.float32)
+        runner = make_tiled_runner(path, 777, tile_size)
+        np.testing.assert_array_equal(gpu_leaf_ids(runner, x), cpu_oracle.leaf_ids(forest, x))
+        np.testing.assert_array_equal(gpu_leaf_ids(runner, x), cpu_oracle.TiledForest(forest, tile_size).leaf_ids(x))
+
+
+@pytest.mark.parametrize("plan", [(64, 1, 1, 16384, 1), (128, 8, 2, 32768, 3), (256, 4, 4, 40960, 2), (64, 16, 2, 24576, 5)])
+@pytest.mark.parametrize("tile_size", [2, 3, 4])
+def test_tiled_launch_plans_agree(synth_model, tile_size, plan):
+    forest = model_io.load_xgboost_json(synth_model(2))
+    x = synth.CONFIGS[2].batch_rows(1501, seed_offset=6)
+    x[3, :] = np.inf
+    x[4, :] = -np.inf
+    x[5, :] = np.nan
+    runner = make_tiled_runner(synth_model(2), 1501, tile_size)
+    runner.set_plan(*plan)
+    assert " tileSize=%d " % tile_size in runner.describe_plan()
+    check_against_oracle(runner, forest, x)
+
+
+def test_tile_sizes_the_kernels_do_not_walk_are_refused(synth_model):
+    with pytest.raises(RuntimeError, match="tile size 8 is not supported"):
+        make_tiled_runner(synth_model(1), 64, 8)
+    with pytest.raises(RuntimeError, match="row tile below 64 KB"):
+        make_tiled_runner(synth_model(4), 64, 2)          # 2000 features: no tiled row tile
+    runner = make_tiled_runner(synth_model(1), 64, 2)
+    with pytest.raises(RuntimeError, match="row-parallel kernel"):
+        runner.set_tree_parallel_plan(4, 64, 1, 0, 1)
+
+
+@pytest.mark.parametrize("tile_size,tiling_type,peel", [(4, 1, True), (4, 2, False), (2, 1, True), (3, 2, True), (1, 1, True)])
+def test_profiled_runner_selects_the_same_leaves(synth_model, plain_file, tmp_path, tile_size, tiling_type, peel):
+    """Probability-based / hybrid tiling and peeled walks change the layout and the trip counts, never the leaf: a
+    profiled and an unprofiled runner agree on configuration 5 (skewed) and on the reference's higgs profile."""
+    forest = model_io.load_xgboost_json(synth_model(5))
+    x = synth.CONFIGS[5].batch_rows(3000, seed_offset=8)
+    profile = write_profile(tmp_path / "c5.profile.csv", forest, cpu_oracle.leaf_ids(forest, synth.CONFIGS[5].batch_rows(4000)))
+    plain = make_tiled_runner(synth_model(5), 3000, tile_size)
+    profiled = make_tiled_runner(synth_model(5), 3000, tile_size, tiling_type, profile, peel)
+    plan = profiled.describe_plan()
+    assert " tiling=%d " % tiling_type in plan and " peelWalks=%d " % int(peel) in plan
+    if tile_size > 1:
+        assert int(plan.split("treesTiledByProfile=")[1].split()[0]) > 0
+    expected = cpu_oracle.leaf_ids(forest, x)
+    np.testing.assert_array_equal(gpu_leaf_ids(profiled, x), expected)
+    np.testing.assert_array_equal(gpu_leaf_ids(plain, x), expected)
+    np.testing.assert_array_equal(gpu_predict(profiled, x), gpu_predict(plain, x))
+    # the reference's own profile of its higgs model
+    higgs = plain_file(benchmark_model("higgs"))
+    higgs_profile = plain_file(os.path.join(GOLDEN, "benchmark", "higgs.test.profile.csv.gz"))
+    data = np.loadtxt(benchmark_csv("higgs"), delimiter=",", dtype=np.float64)
+    hx = data[:, :-1].astype(np.float32)
+    hforest = model_io.load_xgboost_json(higgs)
+    runner = make_tiled_runner(higgs, hx.shape[0], tile_size, tiling_type, higgs_profile, peel)
+    np.testing.assert_array_equal(gpu_leaf_ids(runner, hx), cpu_oracle.leaf_ids(hforest, hx))
+    np.testing.assert_allclose(gpu_predict(runner, hx), data[:, -1], rtol=RTOL_SUM, atol=ATOL_PROB)

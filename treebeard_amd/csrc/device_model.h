@@ -22,6 +22,24 @@
 //  * Trees are walked K at a time (a BUNDLE) to give every lane K independent
 //    dependency chains.  A bundle records the K root addresses, the trip count
 //    (deepest tree of the bundle) and the class the trees add to.
+//
+// Tiled layout (LaunchPlan::tileSize T in {2, 3, 4}; the reference's tile of T connected internal nodes,
+// src/mlir/UniformTilingTransformation.cpp:148-195, src/mlir/ProbabilityBasedTilingTransform.cpp:124-198):
+//  * A TILE holds its nodes in level order, struct-of-arrays: T thresholds, T feature offsets, the byte
+//    address of its first child tile and a child-select table, in 16 / 24 / 32 bytes for T = 2 / 3 / 4:
+//      T = 2: { f32 thr[2]; u16 off[2]; u16 childBase; u16 select }                      one 16-byte read
+//      T = 3: { f32 thr[3]; u16 off[3]; u16 childBase; u16 select; u16 pad }             three 8-byte reads
+//      T = 4: { f32 thr[4]; u16 off[4]; u16 childBase; u16 selectLow; u32 selectHigh }   two 16-byte reads
+//  * The children of a tile (tiles or leaves, numbered left to right as in
+//    docs/TileShapesAndLUT/TileShapesAndLUT.md:23-27) are consecutive tiles, child c at childBase + c * tile
+//    bytes.  `select` is the tile's own row of the reference's LUT[shape][outcome]
+//    (src/utils/TreeTilingUtils.cpp:1932-2018): field number `outcome` (2 bits wide for T <= 3, 3 bits for
+//    T = 4) is the child reached when bit i of `outcome` says that node i's predicate held (node 0 in the
+//    least significant bit, src/mlir/CodeGenStateMachine.cpp:284-506).  Keeping the row in the tile saves the
+//    shape id and the table lookup.
+//  * Unused node slots of a short tile test the pad feature; their outcome bits are don't-cares of `select`.
+//  * A leaf is a tile of its own: thr[0] is the prediction, every slot tests the pad feature, childBase is
+//    the tile's own address and select is 0, so a walk of `depth` tile steps needs no leaf test either.
 #pragma once
 
 #include <cstdint>
@@ -30,6 +48,11 @@ namespace tbamd {
 
 constexpr int kMaxInterleave = 8;
 constexpr uint32_t kNodeBytes = 8;
+constexpr int kMaxTileSize = 4;
+// Bytes of one tile of T nodes (T = 1 is the scalar node).
+constexpr uint32_t TileBytes(int tileSize) { return tileSize <= 1 ? kNodeBytes : tileSize == 2 ? 16u : tileSize == 3 ? 24u : 32u; }
+// Width of one field of a tile's child-select table.
+constexpr uint32_t TileSelectBits(int tileSize) { return tileSize == 4 ? 3u : 2u; }
 
 struct DeviceNode {
   float value;
@@ -38,10 +61,10 @@ struct DeviceNode {
 
 struct alignas(32) DeviceBundle {
   uint16_t root[kMaxInterleave]; // byte address of each tree's root inside the group
-  uint32_t depth;                // walk steps that bring every row to a leaf
+  uint32_t depth;                // walk steps (tile steps in the tiled layout) that bring every row to a leaf
   uint32_t classId;              // (32-bit fields: the kernels fetch a bundle with scalar loads only)
   uint32_t firstSlot;            // index of root[0] in the slot->tree table
-  uint32_t reserved;
+  uint32_t peelDepth;            // steps taken without looking; the rest runs while any lane still moves (== depth: no tail)
 };
 
 // Node of the global-memory walk (trees too big for an LDS group): 16 bytes, absolute indices.

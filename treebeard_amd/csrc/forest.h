@@ -53,6 +53,13 @@ struct Forest {
   void Validate() const;
 };
 
+// Leaf hit counts of a profiling run (the reference's probability profile, src/utils/StatsUtils.cpp:10-52),
+// with the counts of the internal nodes filled in from their subtrees.
+struct HitCountProfile {
+  int64_t numRows = 0;
+  std::vector<std::vector<int64_t>> hits; // per tree, per node
+};
+
 // src/json/xgboostparser.h:117-219
 Forest LoadXGBoostJSON(const std::string &path);
 // src/json/onnxmodelparser.h:50-374; numFeatures comes from CompilerOptions.

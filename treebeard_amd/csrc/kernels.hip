@@ -266,8 +266,10 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
             addr[k] = (root.meta >> 16) + (left ? 0u : kNodeBytes);
           }
         }
+        // bd.peelDepth (== depth unless a hit-count profile asked for peeled walks) steps are taken blind ...
+        const int blind = (int)bd.peelDepth;
 #pragma unroll 2
-        for (int d = kMode != kTileRankU8 ? 1 : 0; d < depth; ++d) {
+        for (int d = kMode != kTileRankU8 ? 1 : 0; d < blind; ++d) {
 #pragma unroll
           for (int k = 0; k < K; ++k) {
             const U32x2 node = LdsLoadNode(addr[k]);
@@ -277,6 +279,228 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
             else left = LdsLoadFloat(column + off) < AsFloat(node.x);
             addr[k] = (node.y >> 16) + (left ? 0u : kNodeBytes);
           }
+        }
+        // ... and the rest only while some lane of the wave still moves (leaves point at themselves)
+        for (int d = blind > 1 || kMode == kTileRankU8 ? blind : 1; d < depth; ++d) {
+          bool moved = false;
+#pragma unroll
+          for (int k = 0; k < K; ++k) {
+            const U32x2 node = LdsLoadNode(addr[k]);
+            const uint32_t off = kMode == kTileF32Bytes ? (node.y & 0xFFFFu) : (node.y & 0xFFFFu) << 2;
+            bool left;
+            if (kMode == kTileRankU8) left = LdsLoadByte(column + off) <= node.x;
+            else left = LdsLoadFloat(column + off) < AsFloat(node.x);
+            const uint32_t next = (node.y >> 16) + (left ? 0u : kNodeBytes);
+            moved = moved || next != addr[k];
+            addr[k] = next;
+          }
+          if (!__any(moved)) break;
+        }
+#pragma unroll
+        for (int k = 0; k < K; ++k) acc += (double)LdsLoadFloat(addr[k]);
+        if (kDump) {
+          if (lane < valid) {
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+              const int tree = slotTree[bd.firstSlot + k];
+              if (tree >= 0) leafIds[row * s.numTrees + tree] = nodeOrigin[grp.nodeBegin + addr[k] / kNodeBytes];
+            }
+          }
+        }
+      }
+      b0 = b1;
+    }
+  }
+
+  if (C > 0) {
+    TBAMD_FLUSH_CLASS(C)
+    return;
+  }
+  if (TT > 1) {
+    __syncthreads();
+    meet[tid] = acc;
+    __syncthreads();
+    if (tt != 0) return;
+    acc = 0.0;
+    for (int t = 0; t < TT; ++t) acc += meet[t * RB + lane];
+  }
+  if (lane >= valid) return;
+  if (partial) {
+    partialRow[0] = acc;
+  } else {
+    const double margin = s.initialValue + acc;
+    out[row] = (float)(s.transform == 1 ? 1.0 / (1.0 + exp(-margin)) : margin);
+  }
+#undef TBAMD_FLUSH_CLASS
+#undef TBAMD_PREFETCH_GROUP
+}
+
+// ---------------------------------------------------------------------------
+// Row-parallel walk over TILED trees (tiles of T = 2, 3 or 4 nodes, layout in device_model.h): the
+// reference's tile step (src/mlir/CodeGenStateMachine.cpp:284-506, cooperative GPU form
+// src/gpu/GPUSimtPass.cpp:39-133) as branch-free per-lane code.  One step reads the tile (thresholds,
+// feature offsets, child base and the tile's own child-select row) with one or two wide LDS reads, gathers
+// the T feature values of the lane's row, turns the T comparisons into an outcome word (node i in bit i)
+// and picks the child out of the select row with one shift.  Leaves are tiles that select themselves, so a
+// bundle walks `depth` tile steps without a leaf test.  Block shape, row tile, tree groups, tree threads,
+// class flush and epilogue are those of WalkRowsLdsKernel.
+//
+// Bundles carry a peel depth (taken from a hit-count profile: the steps that bring 90 % of the profiled
+// rows to a leaf, src/mlir/ProbabilityBasedTilingTransform.cpp:66-73; equal to the depth without one): the
+// walk takes that many steps blind and then goes on only while some lane of the wave still moves, at most to
+// the full depth.
+// ---------------------------------------------------------------------------
+typedef const __attribute__((address_space(3))) U32x4 *LdsQuadPtr;
+__device__ __forceinline__ U32x4 LdsLoadQuad(uint32_t address) { return *(LdsQuadPtr)(uintptr_t)address; }
+
+template <int T>
+__device__ __forceinline__ uint32_t TileStep(uint32_t addr, uint32_t column) {
+  float thr[T];
+  uint32_t off[T];
+  uint32_t childBase;
+  uint64_t select;
+  if (T == 2) {
+    const U32x4 q = LdsLoadQuad(addr);
+    thr[0] = AsFloat(q.x), thr[1] = AsFloat(q.y);
+    off[0] = q.z & 0xFFFFu, off[1] = q.z >> 16;
+    childBase = q.w & 0xFFFFu;
+    select = q.w >> 16;
+  } else if (T == 3) {
+    const U32x2 a = LdsLoadNode(addr), b = LdsLoadNode(addr + 8), c = LdsLoadNode(addr + 16);
+    thr[0] = AsFloat(a.x), thr[1] = AsFloat(a.y), thr[2] = AsFloat(b.x);
+    off[0] = b.y & 0xFFFFu, off[1] = b.y >> 16, off[2] = c.x & 0xFFFFu;
+    childBase = c.x >> 16;
+    select = c.y & 0xFFFFu;
+  } else {
+    const U32x4 q0 = LdsLoadQuad(addr), q1 = LdsLoadQuad(addr + 16);
+    thr[0] = AsFloat(q0.x), thr[1] = AsFloat(q0.y), thr[2] = AsFloat(q0.z), thr[3] = AsFloat(q0.w);
+    off[0] = q1.x & 0xFFFFu, off[1] = q1.x >> 16, off[2] = q1.y & 0xFFFFu, off[3] = q1.y >> 16;
+    childBase = q1.z & 0xFFFFu;
+    select = (uint64_t)(q1.z >> 16) | ((uint64_t)q1.w << 16);
+  }
+  uint32_t outcome = 0;
+#pragma unroll
+  for (int i = 0; i < T; ++i) {
+    const float x = LdsLoadFloat(column + off[i]);
+    outcome |= (x < thr[i] ? 1u : 0u) << i;
+  }
+  const uint32_t child = (uint32_t)(select >> (outcome * TileSelectBits(T))) & ((1u << TileSelectBits(T)) - 1u);
+  return childBase + child * TileBytes(T);
+}
+
+template <int T, int K, int PF, bool kDump>
+__global__ void __launch_bounds__(1024)
+WalkRowsTiledKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16,
+                    const DeviceBundle *__restrict__ bundles, const DeviceGroup *__restrict__ groups,
+                    const WalkScalars s, float *__restrict__ out, double *__restrict__ partial,
+                    int32_t *__restrict__ leafIds, const int32_t *__restrict__ nodeOrigin,
+                    const int32_t *__restrict__ slotTree) {
+  extern __shared__ __align__(16) unsigned char lds[];
+  const int tid = threadIdx.x;
+  const int threads = blockDim.x;
+  const int RB = s.rowsPerBlock;
+  const int TT = s.treeThreads;
+  const int lane = tid & (RB - 1);
+  const int tt = __builtin_amdgcn_readfirstlane(tid / RB);
+  const int F = s.numFeatures;
+  const int64_t row0 = (int64_t)blockIdx.x * RB;
+  const int64_t remaining = s.rows - row0;
+  const int valid = remaining < RB ? (int)remaining : RB;
+
+  float *rowTile = reinterpret_cast<float *>(lds + s.groupRegionBytes);
+  StageRows<true>(x + row0 * F, valid, RB, F, 0, rowTile, tid, threads);
+  for (int i = tid; i < RB; i += threads) rowTile[F * RB + i] = -INFINITY; // pad feature: keeps leaves in place
+  const uint32_t column = s.groupRegionBytes + (uint32_t)lane * 4u;
+
+  const int slice = blockIdx.y;
+  const int gBegin = (int)(((int64_t)s.numGroups * slice) / s.treeSlices);
+  const int gEnd = (int)(((int64_t)s.numGroups * (slice + 1)) / s.treeSlices);
+  const int C = s.numClasses;
+  const int64_t row = row0 + lane;
+  double *partialRow = partial ? partial + ((int64_t)slice * s.rows + row) * (C > 0 ? C : 1) : nullptr;
+  double *meet = reinterpret_cast<double *>(C > 0 ? lds + ((s.groupRegionBytes + (uint32_t)(F + 1) * RB * 4u + 7u) & ~7u) : lds);
+
+  double acc = 0.0;
+  int curClass = 0;
+  U32x4 fetched[PF];
+#define TBAMD_PREFETCH_GROUP(NEXTGRP)                                                                                  \
+  {                                                                                                                    \
+    const DeviceGroup nextGrp = (NEXTGRP);                                                                             \
+    const U32x4 *src = reinterpret_cast<const U32x4 *>(nodes16) + (nextGrp.nodeBegin >> 1);                            \
+    const int last = (int)(nextGrp.nodeCount >> 1) - 1;                                                                \
+    _Pragma("unroll") for (int i = 0; i < PF; ++i) {                                                                   \
+      const int idx = tid + i * threads;                                                                               \
+      fetched[i] = src[idx < last ? idx : last];                                                                       \
+    }                                                                                                                  \
+  }
+#define TBAMD_FLUSH_CLASS(UPTO)                                                                                        \
+  {                                                                                                                    \
+    if (TT > 1) {                                                                                                      \
+      __syncthreads();                                                                                                 \
+      meet[tid] = acc;                                                                                                 \
+      __syncthreads();                                                                                                 \
+      if (tt == 0) {                                                                                                   \
+        acc = 0.0;                                                                                                     \
+        for (int t = 0; t < TT; ++t) acc += meet[t * RB + lane];                                                       \
+      }                                                                                                                \
+    }                                                                                                                  \
+    if (tt == 0 && lane < valid) {                                                                                     \
+      partialRow[curClass] = acc;                                                                                      \
+      for (int c = curClass + 1; c < (UPTO); ++c) partialRow[c] = 0.0;                                                 \
+    }                                                                                                                  \
+    acc = 0.0;                                                                                                         \
+  }
+  if (gBegin < gEnd) TBAMD_PREFETCH_GROUP(groups[gBegin])
+
+  for (int g = gBegin; g < gEnd; ++g) {
+    const DeviceGroup grp = groups[g];
+    __syncthreads();
+    {
+      U32x4 *dst = reinterpret_cast<U32x4 *>(lds);
+      const int pieces = (int)(grp.nodeCount >> 1);
+#pragma unroll
+      for (int i = 0; i < PF; ++i) {
+        const int idx = tid + i * threads;
+        if (idx < pieces) dst[idx] = fetched[i];
+      }
+    }
+    __syncthreads();
+    if (g + 1 < gEnd) TBAMD_PREFETCH_GROUP(groups[g + 1])
+
+    uint32_t b0 = 0;
+    while (b0 < grp.bundleCount) {
+      uint32_t b1 = grp.bundleCount;
+      if (C > 0) {
+        const int cls = grp.uniformClass ? (int)grp.uniformClass - 1 : (int)bundles[grp.bundleBegin + b0].classId;
+        if (cls != curClass) {
+          TBAMD_FLUSH_CLASS(cls)
+          curClass = cls;
+        }
+        if (!grp.uniformClass) {
+          b1 = b0 + 1;
+          while (b1 < grp.bundleCount && (int)bundles[grp.bundleBegin + b1].classId == cls) ++b1;
+        }
+      }
+      for (uint32_t b = b0 + tt; b < b1; b += TT) {
+        const DeviceBundle bd = bundles[grp.bundleBegin + b];
+        uint32_t addr[K];
+#pragma unroll
+        for (int k = 0; k < K; ++k) addr[k] = bd.root[k];
+        const int depth = (int)bd.depth;
+        const int blind = (int)bd.peelDepth;
+        for (int d = 0; d < blind; ++d) {
+#pragma unroll
+          for (int k = 0; k < K; ++k) addr[k] = TileStep<T>(addr[k], column);
+        }
+        for (int d = blind; d < depth; ++d) {
+          bool moved = false;
+#pragma unroll
+          for (int k = 0; k < K; ++k) {
+            const uint32_t next = TileStep<T>(addr[k], column);
+            moved = moved || next != addr[k];
+            addr[k] = next;
+          }
+          if (!__any(moved)) break; // every lane of the wave sits on a leaf tile (leaves select themselves)
         }
 #pragma unroll
         for (int k = 0; k < K; ++k) acc += (double)LdsLoadFloat(addr[k]);
@@ -795,6 +1019,61 @@ hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, int tileMode, 
   case kTileRankU8:
     if (RB != 64) return hipErrorInvalidValue;
     return LaunchWalkW<kTileRankU8>(p, interleave, prefetch, grid, block, ldsBytes, stream);
+  default: return hipErrorInvalidValue;
+  }
+}
+
+namespace {
+template <int T, int K, int PF>
+hipError_t LaunchTiledTKP(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
+  if (p.leafIds) {
+    hipError_t e = AllowFullLds<&WalkRowsTiledKernel<T, K, PF, true>>();
+    if (e != hipSuccess) return e;
+    WalkRowsTiledKernel<T, K, PF, true><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out, p.partial,
+                                                                          p.leafIds, p.nodeOrigin, p.slotTree);
+  } else {
+    hipError_t e = AllowFullLds<&WalkRowsTiledKernel<T, K, PF, false>>();
+    if (e != hipSuccess) return e;
+    WalkRowsTiledKernel<T, K, PF, false><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out, p.partial,
+                                                                           nullptr, nullptr, nullptr);
+  }
+  return hipGetLastError();
+}
+
+template <int T, int K>
+hipError_t LaunchTiledTK(const WalkParams &p, int prefetch, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
+  if (prefetch <= 4) return LaunchTiledTKP<T, K, 4>(p, grid, block, ldsBytes, stream);
+  if (prefetch <= 8) return LaunchTiledTKP<T, K, 8>(p, grid, block, ldsBytes, stream);
+  if (prefetch <= 16) return LaunchTiledTKP<T, K, 16>(p, grid, block, ldsBytes, stream);
+  return hipErrorInvalidValue;
+}
+
+template <int T>
+hipError_t LaunchTiledT(const WalkParams &p, int interleave, int prefetch, dim3 grid, dim3 block, size_t ldsBytes,
+                        hipStream_t stream) {
+  switch (interleave) {
+  case 1: return LaunchTiledTK<T, 1>(p, prefetch, grid, block, ldsBytes, stream);
+  case 2: return LaunchTiledTK<T, 2>(p, prefetch, grid, block, ldsBytes, stream);
+  case 4: return LaunchTiledTK<T, 4>(p, prefetch, grid, block, ldsBytes, stream);
+  default: return hipErrorInvalidValue;
+  }
+}
+} // namespace
+
+hipError_t LaunchWalkRowsTiled(const WalkParams &p, int tileSize, int interleave, size_t ldsBytes, hipStream_t stream) {
+  if (p.s.rows <= 0) return hipSuccess;
+  const int RB = p.s.rowsPerBlock, TT = p.s.treeThreads;
+  if (ldsBytes > 160 * 1024 || RB < 64 || (RB & (RB - 1)) || TT < 1 || RB * TT > 1024) return hipErrorInvalidValue;
+  // feature offsets are byte offsets into the f32 row tile: the tile has to end below 64 KB
+  if ((int64_t)(p.s.numFeatures + 1) * RB * 4 > 0x10000) return hipErrorInvalidValue;
+  const int64_t blocks = (p.s.rows + RB - 1) / RB;
+  if (blocks > 0x7FFFFFFF || p.s.treeSlices < 1 || p.s.treeSlices > 65535) return hipErrorInvalidValue;
+  const int prefetch = (int)((p.s.groupRegionBytes / 16 + RB * TT - 1) / (RB * TT));
+  dim3 grid((unsigned)blocks, (unsigned)p.s.treeSlices), block((unsigned)(RB * TT));
+  switch (tileSize) {
+  case 2: return LaunchTiledT<2>(p, interleave, prefetch, grid, block, ldsBytes, stream);
+  case 3: return LaunchTiledT<3>(p, interleave, prefetch, grid, block, ldsBytes, stream);
+  case 4: return LaunchTiledT<4>(p, interleave, prefetch, grid, block, ldsBytes, stream);
   default: return hipErrorInvalidValue;
   }
 }

@@ -21,7 +21,7 @@ namespace tbamd {
 namespace {
 
 constexpr char kMagic[8] = {'T', 'B', 'A', 'M', 'D', 'M', 'D', 'L'};
-constexpr uint32_t kVersion = 2;
+constexpr uint32_t kVersion = 3;
 
 struct Writer {
   std::string bytes;
@@ -55,7 +55,7 @@ struct Reader {
 } // namespace
 
 void SaveCompiledModel(const std::string &path, const Forest &forest, const LaunchPlan &plan, int32_t batchSize,
-                       int32_t returnTypeWidth, bool returnTypeFloatType) {
+                       int32_t returnTypeWidth, bool returnTypeFloatType, const HitCountProfile *profile) {
   Writer w;
   w.bytes.append(kMagic, sizeof(kMagic));
   w.Put<uint32_t>(kVersion);
@@ -76,6 +76,9 @@ void SaveCompiledModel(const std::string &path, const Forest &forest, const Laun
   w.Put<int32_t>(plan.treeSlices);
   w.Put<int32_t>(plan.featureOffsetInWords ? 1 : 0);
   w.Put<int32_t>(plan.quantizedRows ? 1 : 0);
+  w.Put<int32_t>(plan.tileSize);
+  w.Put<int32_t>(plan.tiling);
+  w.Put<int32_t>(plan.peelWalks ? 1 : 0);
   w.Put<uint64_t>(forest.trees.size());
   for (const Tree &t : forest.trees) {
     w.Put<int32_t>(t.classId);
@@ -84,6 +87,9 @@ void SaveCompiledModel(const std::string &path, const Forest &forest, const Laun
     w.PutVector(t.left);
     w.PutVector(t.right);
   }
+  w.Put<int64_t>(profile ? profile->numRows : -1);
+  if (profile)
+    for (const auto &hits : profile->hits) w.PutVector(hits);
   std::ofstream out(path, std::ios::binary | std::ios::trunc);
   if (!out) throw Error("cannot write " + path);
   out.write(w.bytes.data(), (std::streamsize)w.bytes.size());
@@ -114,6 +120,9 @@ CompiledModel LoadCompiledModel(const std::string &path) {
   m.plan.treeSlices = r.Get<int32_t>();
   m.plan.featureOffsetInWords = r.Get<int32_t>() != 0;
   m.plan.quantizedRows = r.Get<int32_t>() != 0;
+  m.plan.tileSize = r.Get<int32_t>();
+  m.plan.tiling = r.Get<int32_t>();
+  m.plan.peelWalks = r.Get<int32_t>() != 0;
   const uint64_t trees = r.Get<uint64_t>();
   if (trees > bytes.size()) throw Error("model file is truncated");
   m.forest.trees.resize(trees);
@@ -125,6 +134,16 @@ CompiledModel LoadCompiledModel(const std::string &path) {
     t.right = r.GetVector<int32_t>();
   }
   m.forest.Validate();
+  const int64_t profileRows = r.Get<int64_t>();
+  if (profileRows >= 0) {
+    m.profile = std::make_unique<HitCountProfile>();
+    m.profile->numRows = profileRows;
+    m.profile->hits.resize(trees);
+    for (size_t t = 0; t < trees; ++t) {
+      m.profile->hits[t] = r.GetVector<int64_t>();
+      if (m.profile->hits[t].size() != m.forest.trees[t].NumNodes()) throw Error("model file: profile does not match the forest");
+    }
+  }
   return m;
 }
 

@@ -3,6 +3,7 @@
 #include "forest.h"
 #include "packer.h"
 
+#include <memory>
 #include <string>
 #include <vector>
 
@@ -14,18 +15,12 @@ struct CompiledModel {
   int32_t batchSize = 0;
   int32_t returnTypeWidth = 32;
   bool returnTypeFloatType = true;
+  std::unique_ptr<HitCountProfile> profile; // the hit counts the model was tiled with, if any
 };
 
 void SaveCompiledModel(const std::string &path, const Forest &forest, const LaunchPlan &plan, int32_t batchSize,
-                       int32_t returnTypeWidth, bool returnTypeFloatType);
+                       int32_t returnTypeWidth, bool returnTypeFloatType, const HitCountProfile *profile = nullptr);
 CompiledModel LoadCompiledModel(const std::string &path);
-
-// Leaf hit counts of a profiling run (the reference's probability profile), with the counts of the
-// internal nodes filled in from their subtrees.
-struct HitCountProfile {
-  int64_t numRows = 0;
-  std::vector<std::vector<int64_t>> hits; // per tree, per node
-};
 
 HitCountProfile LoadHitCountProfile(const Forest &forest, const std::string &path);
 // Average number of internal nodes a profiled row visits over the whole forest.

@@ -2,6 +2,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <functional>
 #include <limits>
 #include <cstring>
 #include <numeric>
@@ -92,6 +93,253 @@ LevelOrder MakeLevelOrder(const Tree &tree) {
 
 } // namespace
 
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// Tiling of one tree (LaunchPlan::tileSize > 1).
+// ---------------------------------------------------------------------------
+struct TileInfo {
+  int32_t count = 0;                       // internal nodes in the tile; 0: a leaf tile
+  int32_t members[kMaxTileSize] = {};      // original node ids, level order inside the tile
+  int32_t numExits = 0;
+  int32_t exits[kMaxTileSize + 1] = {};    // original node ids the tile's children start at, left to right
+  int32_t leafNode = -1;                   // leaf tiles: the original leaf
+  uint32_t firstChild = 0;                 // tile index (inside the tree) of child 0; own index on a leaf tile
+  uint64_t select = 0;                     // child number per outcome word, TileSelectBits() each
+  int32_t depth = 0;                       // tile steps from this tile down to its deepest leaf
+  int32_t level = 0;                       // tile steps from the root tile
+};
+
+struct TiledTree {
+  std::vector<TileInfo> tiles; // children of a tile are consecutive
+  int32_t depth = 0;           // tile steps that bring every row to a leaf tile
+  bool byProfile = false;
+};
+
+// Members of the tile rooted at `root`, breadth first over internal nodes, left before right
+// (src/mlir/UniformTilingTransformation.cpp:148-168).
+int GatherUniform(const Tree &tree, int32_t root, int T, int32_t *members) {
+  int32_t queue[2 * kMaxTileSize + 2];
+  int head = 0, tail = 0, n = 0;
+  queue[tail++] = root;
+  while (head < tail && n < T) {
+    const int32_t node = queue[head++];
+    members[n++] = node;
+    if (!tree.IsLeaf(tree.left[node])) queue[tail++] = tree.left[node];
+    if (!tree.IsLeaf(tree.right[node])) queue[tail++] = tree.right[node];
+  }
+  return n;
+}
+
+// Members chosen by visit counts: the tile grows by the most-visited internal child of any member
+// (src/mlir/ProbabilityBasedTilingTransform.cpp:152-190: members are scanned in node order, left child before
+// right, and a candidate wins only with strictly more hits).
+int GatherByHits(const Tree &tree, const std::vector<int64_t> &hits, int32_t root, int T, int32_t *members) {
+  int n = 0;
+  members[n++] = root;
+  while (n < T) {
+    int32_t sorted[kMaxTileSize];
+    std::copy(members, members + n, sorted);
+    std::sort(sorted, sorted + n);
+    int64_t bestHits = -1;
+    int32_t best = -1;
+    for (int i = 0; i < n; ++i)
+      for (int32_t child : {tree.left[sorted[i]], tree.right[sorted[i]]}) {
+        if (tree.IsLeaf(child) || hits[child] <= bestHits) continue;
+        if (std::find(members, members + n, child) != members + n) continue;
+        bestHits = hits[child];
+        best = child;
+      }
+    if (best < 0) break;
+    members[n++] = best;
+  }
+  return n;
+}
+
+// src/mlir/ProbabilityBasedTilingTransform.cpp:208-225: the most-visited tenth of the leaves takes more
+// than 90 % of the rows.
+bool IsSkewed(const Tree &tree, const std::vector<int64_t> &hits) {
+  std::vector<int64_t> leafHits;
+  for (size_t i = 0; i < tree.NumNodes(); ++i)
+    if (tree.IsLeaf((int32_t)i)) leafHits.push_back(hits[i]);
+  std::sort(leafHits.begin(), leafHits.end(), std::greater<int64_t>());
+  const size_t consider = (size_t)((double)leafHits.size() * 0.10);
+  int64_t covered = 0;
+  for (size_t i = 0; i < consider; ++i) covered += leafHits[i];
+  return hits[0] > 0 && (double)covered / (double)hits[0] > 0.9;
+}
+
+TiledTree TileTree(const Tree &tree, int T, int tiling, const std::vector<int64_t> *hits) {
+  TiledTree out;
+  out.byProfile = tiling != 0 && hits != nullptr && IsSkewed(tree, *hits);
+  // depth of every original node, for the level order inside a tile
+  std::vector<int32_t> nodeDepth(tree.NumNodes(), -1);
+  {
+    std::vector<int32_t> stack{0};
+    nodeDepth[0] = 0;
+    while (!stack.empty()) {
+      const int32_t n = stack.back();
+      stack.pop_back();
+      if (tree.IsLeaf(n)) continue;
+      nodeDepth[tree.left[n]] = nodeDepth[tree.right[n]] = nodeDepth[n] + 1;
+      stack.push_back(tree.left[n]);
+      stack.push_back(tree.right[n]);
+    }
+  }
+  std::vector<int32_t> roots{0}; // node each tile starts at, in tile order
+  for (size_t ti = 0; ti < roots.size(); ++ti) {
+    TileInfo tile;
+    const int32_t root = roots[ti];
+    if (tree.IsLeaf(root)) {
+      tile.leafNode = root;
+      tile.firstChild = (uint32_t)ti;
+      out.tiles.push_back(tile);
+      continue;
+    }
+    bool byHits = out.byProfile;
+    if (byHits && tiling == 2 && (double)(*hits)[root] / (double)(*hits)[0] < 0.20) byHits = false; // hybrid
+    int32_t members[kMaxTileSize];
+    const int n = byHits ? GatherByHits(tree, *hits, root, T, members) : GatherUniform(tree, root, T, members);
+    // level order inside the tile: by depth, then left to right (position in an in-order walk of the tile)
+    std::vector<int32_t> inorder;
+    {
+      // in-order walk restricted to the members
+      std::vector<std::pair<int32_t, int>> stack{{root, 0}};
+      while (!stack.empty()) {
+        auto [node, state] = stack.back();
+        stack.pop_back();
+        const bool member = std::find(members, members + n, node) != members + n;
+        if (!member) continue;
+        if (state == 0) {
+          stack.push_back({node, 1});
+          stack.push_back({tree.left[node], 0});
+        } else {
+          inorder.push_back(node);
+          stack.push_back({tree.right[node], 0});
+        }
+      }
+    }
+    std::vector<int32_t> ordered(members, members + n);
+    std::stable_sort(ordered.begin(), ordered.end(), [&](int32_t a, int32_t b) {
+      if (nodeDepth[a] != nodeDepth[b]) return nodeDepth[a] < nodeDepth[b];
+      return std::find(inorder.begin(), inorder.end(), a) < std::find(inorder.begin(), inorder.end(), b);
+    });
+    tile.count = n;
+    std::copy(ordered.begin(), ordered.end(), tile.members);
+    // tile-local children (slot or -(exit number) - 1), exits numbered left to right
+    int32_t leftSlot[kMaxTileSize], rightSlot[kMaxTileSize];
+    auto slotOf = [&](int32_t node) {
+      for (int i = 0; i < n; ++i)
+        if (tile.members[i] == node) return i;
+      return -1;
+    };
+    {
+      std::vector<std::pair<int, int>> stack{{0, 0}};
+      while (!stack.empty()) {
+        auto [slot, state] = stack.back();
+        stack.pop_back();
+        const int32_t node = tile.members[slot];
+        if (state == 0) {
+          stack.push_back({slot, 1});
+          const int child = slotOf(tree.left[node]);
+          if (child >= 0) {
+            leftSlot[slot] = child;
+            stack.push_back({child, 0});
+          } else {
+            leftSlot[slot] = -(tile.numExits) - 1;
+            tile.exits[tile.numExits++] = tree.left[node];
+          }
+        } else {
+          const int child = slotOf(tree.right[node]);
+          if (child >= 0) {
+            rightSlot[slot] = child;
+            stack.push_back({child, 0});
+          } else {
+            rightSlot[slot] = -(tile.numExits) - 1;
+            tile.exits[tile.numExits++] = tree.right[node];
+          }
+        }
+      }
+    }
+    // the tile's row of the child look-up table: outcome bit i set = node i sends the row left
+    const uint32_t width = TileSelectBits(T);
+    for (uint32_t outcome = 0; outcome < (1u << T); ++outcome) {
+      int slot = 0;
+      for (;;) {
+        const int32_t next = ((outcome >> slot) & 1u) ? leftSlot[slot] : rightSlot[slot];
+        if (next < 0) {
+          tile.select |= (uint64_t)(-next - 1) << (outcome * width);
+          break;
+        }
+        slot = next;
+      }
+    }
+    tile.firstChild = (uint32_t)roots.size();
+    for (int e = 0; e < tile.numExits; ++e) roots.push_back(tile.exits[e]);
+    out.tiles.push_back(tile);
+  }
+  // levels top down (children follow their parent in tile order), depths bottom up
+  for (size_t ti = 0; ti < out.tiles.size(); ++ti)
+    for (int e = 0; e < out.tiles[ti].numExits; ++e)
+      out.tiles[out.tiles[ti].firstChild + e].level = out.tiles[ti].level + 1;
+  for (size_t ti = out.tiles.size(); ti-- > 0;) {
+    TileInfo &tile = out.tiles[ti];
+    for (int e = 0; e < tile.numExits; ++e) tile.depth = std::max(tile.depth, 1 + out.tiles[tile.firstChild + e].depth);
+  }
+  out.depth = out.tiles[0].depth;
+  return out;
+}
+
+// Bytes of one tile (see device_model.h) for a tree whose tile 0 sits at byte address `treeBase` of its group.
+void EmitTile(const Tree &tree, const TileInfo &tile, int T, uint32_t treeBase, size_t tileIndex, uint32_t featureStride,
+              uint32_t padOffset, unsigned char *dst) {
+  const uint32_t bytes = TileBytes(T);
+  float thr[kMaxTileSize] = {};
+  uint16_t off[kMaxTileSize];
+  for (int i = 0; i < T; ++i) off[i] = (uint16_t)padOffset;
+  if (tile.count == 0) {
+    thr[0] = tree.value[tile.leafNode];
+  } else {
+    for (int i = 0; i < tile.count; ++i) {
+      thr[i] = tree.value[tile.members[i]];
+      off[i] = (uint16_t)((uint32_t)tree.feature[tile.members[i]] * featureStride);
+    }
+  }
+  const uint32_t childAddress = treeBase + tile.firstChild * bytes;
+  if (childAddress + (uint32_t)std::max(tile.numExits, 1) * bytes > 0x10000u) throw Error("internal error: tile address beyond the group");
+  const uint16_t childBase = (uint16_t)childAddress;
+  std::memset(dst, 0, bytes);
+  std::memcpy(dst, thr, (size_t)T * 4);
+  std::memcpy(dst + T * 4, off, (size_t)T * 2);
+  std::memcpy(dst + T * 6, &childBase, 2);
+  if (T == 4) {
+    const uint16_t low = (uint16_t)(tile.select & 0xFFFFu);
+    const uint32_t high = (uint32_t)(tile.select >> 16);
+    std::memcpy(dst + 26, &low, 2);
+    std::memcpy(dst + 28, &high, 4);
+  } else {
+    const uint16_t select = (uint16_t)tile.select;
+    std::memcpy(dst + T * 6 + 2, &select, 2);
+  }
+  (void)tileIndex;
+}
+
+// Steps after which 90 % of the profiled rows of a tree have reached their leaf
+// (src/utils/TreeTilingUtils.cpp:1722-1743); `leafLevel[i]` is the step count of leaf i, -1 for other nodes.
+int32_t PeelDepth(const std::vector<int64_t> &hits, const std::vector<int32_t> &leafLevel, int32_t depth) {
+  if (hits.empty() || hits[0] <= 0) return depth;
+  for (int32_t d = 0; d <= depth; ++d) {
+    int64_t covered = 0;
+    for (size_t i = 0; i < leafLevel.size(); ++i)
+      if (leafLevel[i] >= 0 && leafLevel[i] <= d) covered += hits[i];
+    if ((double)covered / (double)hits[0] >= 0.9) return d;
+  }
+  return depth;
+}
+
+} // namespace
+
 namespace {
 
 // Global-memory layout: every tree breadth first (siblings adjacent), absolute node indices.
@@ -140,9 +388,13 @@ PackedModel PackForGlobalWalk(const Forest &forest, const LaunchPlan &plan) {
 
 } // namespace
 
-PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
+PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCountProfile *profile) {
   const Forest forest = NormalizeToLessThan(input);
-  if (plan.kernel == LaunchPlan::Kernel::kGlobalWalk) return PackForGlobalWalk(forest, plan);
+  if (profile && profile->hits.size() != forest.trees.size()) throw Error("hit-count profile does not match the forest");
+  if (plan.kernel == LaunchPlan::Kernel::kGlobalWalk) {
+    if (plan.tileSize > 1) throw Error("tile sizes above 1 need the row-parallel LDS kernel; this forest has a tree too big for LDS");
+    return PackForGlobalWalk(forest, plan);
+  }
   const int K = plan.interleave;
   if (K < 1 || K > kMaxInterleave || (K & (K - 1))) throw Error("interleave must be 1, 2, 4 or 8");
   if (plan.kernel == LaunchPlan::Kernel::kRowParallelLds) {
@@ -162,6 +414,14 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
 
   if (plan.quantizedRows && (plan.kernel != LaunchPlan::Kernel::kRowParallelLds || plan.rowsPerBlock != 64))
     throw Error("rank-quantised rows need the row-parallel kernel with 64 rows per block");
+  const int T = plan.tileSize;
+  if (T < 1 || T > kMaxTileSize)
+    throw Error("tile size " + std::to_string(T) + " is not supported: the device kernels walk tiles of 1 to " +
+                std::to_string(kMaxTileSize) + " nodes");
+  if (T > 1 && (plan.kernel != LaunchPlan::Kernel::kRowParallelLds || plan.quantizedRows))
+    throw Error("tile sizes above 1 need the row-parallel kernel on float32 rows");
+  if (T > 1 && (plan.featureOffsetInWords || (int64_t)(forest.numFeatures + 1) * plan.rowsPerBlock * 4 > 0x10000))
+    throw Error("tile sizes above 1 need a row tile below 64 KB (tiles hold byte offsets): fewer rows per block");
 
   PackedModel pm;
   pm.plan = plan;
@@ -172,7 +432,8 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
   if (padOffset > 0xFFFFu)
     throw Error("feature offsets do not fit 16 bits for this rowsPerBlock / feature count");
   const uint32_t featureStride = plan.FeatureStride();
-  const uint32_t groupCapacity = (uint32_t)plan.groupBytes / kNodeBytes;
+  const uint32_t groupCapacity = (uint32_t)plan.groupBytes / kNodeBytes; // in 8-byte units
+  const uint32_t tileUnits = TileBytes(T) / kNodeBytes;                    // units per tile (1 for scalar nodes)
 
   // Rank quantisation: x < t_j  <=>  #{t : t <= x} <= j for the sorted distinct thresholds t_0 < t_1 < ...
   // of the feature, so an internal node stores j and the kernel compares the row's one-byte rank with it.
@@ -195,27 +456,89 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
         pm.binThresholds[((size_t)(f / chunk) * depth + k) * chunk + (f % chunk)] = ranks[f][k];
   }
 
+  // Per tree: its size in the packed layout, the steps of a lock-step walk, and the steps after which the walk
+  // starts looking whether any lane still moves (walk peeling; equal to the depth when there is no tail).
+  const size_t numTrees = forest.trees.size();
+  std::vector<TiledTree> tiled(T > 1 ? numTrees : 0);
+  std::vector<int32_t> depth(numTrees), peel(numTrees);
+  std::vector<uint32_t> units(numTrees);
+  for (size_t t = 0; t < numTrees; ++t) {
+    const Tree &tree = forest.trees[t];
+    const std::vector<int64_t> *hits = profile ? &profile->hits[t] : nullptr;
+    std::vector<int32_t> leafLevel(tree.NumNodes(), -1);
+    if (T > 1) {
+      tiled[t] = TileTree(tree, T, plan.tiling, hits);
+      depth[t] = tiled[t].depth;
+      units[t] = (uint32_t)tiled[t].tiles.size() * tileUnits;
+      pm.treesTiledByProfile += tiled[t].byProfile ? 1 : 0;
+      for (const TileInfo &tile : tiled[t].tiles)
+        if (tile.count == 0) leafLevel[tile.leafNode] = tile.level;
+    } else {
+      depth[t] = tree.Depth();
+      units[t] = (uint32_t)tree.NumNodes();
+      std::vector<int32_t> stack{0};
+      leafLevel[0] = 0;
+      while (!stack.empty()) { // (the level of every node; only the leaves' entries are used)
+        const int32_t n = stack.back();
+        stack.pop_back();
+        if (tree.IsLeaf(n)) continue;
+        leafLevel[tree.left[n]] = leafLevel[tree.right[n]] = leafLevel[n] + 1;
+        stack.push_back(tree.left[n]);
+        stack.push_back(tree.right[n]);
+      }
+      for (size_t i = 0; i < tree.NumNodes(); ++i)
+        if (!tree.IsLeaf((int32_t)i)) leafLevel[i] = -1;
+    }
+    peel[t] = plan.peelWalks && hits ? PeelDepth(*hits, leafLevel, depth[t]) : depth[t];
+    pm.lockStepSteps += depth[t];
+    if (hits && (*hits)[0] > 0) {
+      double steps = 0.0;
+      for (size_t i = 0; i < tree.NumNodes(); ++i)
+        if (leafLevel[i] >= 0) steps += (double)(*hits)[i] * leafLevel[i];
+      pm.profiledSteps += steps / (double)(*hits)[0];
+    }
+  }
+
   // Order: class, then depth (the reference sorts by depth for its GPU schedules,
   // src/mlir/GPUAutoSchedule.cpp:115-122); stable so equal keys keep model order.
-  std::vector<int32_t> depth(forest.trees.size());
-  for (size_t t = 0; t < forest.trees.size(); ++t) depth[t] = forest.trees[t].Depth();
-  std::vector<int32_t> order(forest.trees.size());
+  std::vector<int32_t> order(numTrees);
   std::iota(order.begin(), order.end(), 0);
   std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) {
     int32_t ca = forest.numClasses > 0 ? forest.trees[a].classId : 0;
     int32_t cb = forest.numClasses > 0 ? forest.trees[b].classId : 0;
     if (ca != cb) return ca < cb;
-    return depth[a] < depth[b];
+    if (depth[a] != depth[b]) return depth[a] < depth[b];
+    return peel[a] < peel[b];
   });
 
+  // The null leaf that padding trees of a bundle point at: a leaf of value 0 at address 0 of every group.
+  auto pushNullLeaf = [&]() {
+    if (T > 1) {
+      Tree nullTree;
+      nullTree.value = {0.0f};
+      nullTree.feature = {0};
+      nullTree.left = nullTree.right = {-1};
+      TileInfo leaf;
+      leaf.leafNode = 0;
+      std::vector<unsigned char> bytes(TileBytes(T));
+      EmitTile(nullTree, leaf, T, 0, 0, featureStride, (uint32_t)padOffset, bytes.data());
+      for (uint32_t u = 0; u < tileUnits; ++u) {
+        DeviceNode unit;
+        std::memcpy(&unit, bytes.data() + u * kNodeBytes, kNodeBytes);
+        pm.nodes.push_back(unit);
+        pm.nodeOrigin.push_back(-1);
+      }
+    } else {
+      pm.nodes.push_back(DeviceNode{0.0f, (0u << 16) | (uint32_t)padOffset});
+      pm.nodeOrigin.push_back(-1);
+    }
+  };
   auto openGroup = [&]() {
     DeviceGroup g{};
     g.nodeBegin = (uint32_t)pm.nodes.size();
     g.bundleBegin = (uint32_t)pm.bundles.size();
     pm.groups.push_back(g);
-    // node 0 of every group: the null leaf padding trees point at
-    pm.nodes.push_back(DeviceNode{0.0f, (0u << 16) | (uint32_t)padOffset});
-    pm.nodeOrigin.push_back(-1);
+    pushNullLeaf();
   };
   auto closeGroup = [&]() {
     DeviceGroup &g = pm.groups.back();
@@ -234,12 +557,52 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
     }
     pm.maxGroupNodes = std::max(pm.maxGroupNodes, g.nodeCount);
   };
+  // Writes tree t with its first unit at unit `base` of the current group.
+  auto emitTree = [&](int32_t t, uint32_t base) {
+    const Tree &tree = forest.trees[t];
+    if (T > 1) {
+      std::vector<unsigned char> bytes(TileBytes(T));
+      for (size_t ti = 0; ti < tiled[t].tiles.size(); ++ti) {
+        const TileInfo &tile = tiled[t].tiles[ti];
+        EmitTile(tree, tile, T, base * kNodeBytes, ti, featureStride, (uint32_t)padOffset, bytes.data());
+        for (uint32_t u = 0; u < tileUnits; ++u) {
+          DeviceNode unit;
+          std::memcpy(&unit, bytes.data() + u * kNodeBytes, kNodeBytes);
+          pm.nodes.push_back(unit);
+          pm.nodeOrigin.push_back(u == 0 ? (tile.count == 0 ? tile.leafNode : tile.members[0]) : -1);
+        }
+      }
+      return;
+    }
+    const LevelOrder lo = MakeLevelOrder(tree);
+    for (size_t i = 0; i < lo.order.size(); ++i) {
+      const int32_t n = lo.order[i];
+      DeviceNode dn;
+      dn.value = tree.value[n];
+      if (plan.quantizedRows && !tree.IsLeaf(n)) {
+        const auto &sorted = ranks[(size_t)tree.feature[n]];
+        const uint32_t j = (uint32_t)(std::lower_bound(sorted.begin(), sorted.end(), tree.value[n]) - sorted.begin());
+        static_assert(sizeof(float) == sizeof(uint32_t), "node value holds the rank bit pattern");
+        std::memcpy(&dn.value, &j, sizeof(j));
+      }
+      if (tree.IsLeaf(n)) {
+        dn.meta = (((base + (uint32_t)i) * kNodeBytes) << 16) | (uint32_t)padOffset;
+      } else {
+        const uint32_t child = base + (uint32_t)lo.position[tree.left[n]];
+        if (lo.position[tree.right[n]] != lo.position[tree.left[n]] + 1)
+          throw Error("internal error: siblings not adjacent");
+        dn.meta = ((child * kNodeBytes) << 16) | ((uint32_t)tree.feature[n] * featureStride);
+      }
+      pm.nodes.push_back(dn);
+      pm.nodeOrigin.push_back(n);
+    }
+  };
 
   size_t next = 0;
   while (next < order.size()) {
     openGroup();
     DeviceGroup &g = pm.groups.back();
-    // one spare node keeps room for the alignment pad
+    // one spare unit keeps room for the alignment pad
     auto freeNodes = [&]() { return groupCapacity - 1 - ((uint32_t)pm.nodes.size() - g.nodeBegin); };
     bool any = false;
     struct Mark { size_t nodes, slots, next; };
@@ -252,13 +615,13 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
       uint32_t need = 0;
       int count = 0;
       while (count < K && next + count < order.size()) {
-        const Tree &tree = forest.trees[order[next + count]];
-        const int32_t c = forest.numClasses > 0 ? tree.classId : 0;
+        const int32_t t = order[next + count];
+        const int32_t c = forest.numClasses > 0 ? forest.trees[t].classId : 0;
         if (c != cls) break;
-        if ((uint32_t)tree.NumNodes() + 2 > groupCapacity)
-          throw Error("a tree of " + std::to_string(tree.NumNodes()) + " nodes does not fit one LDS tree group");
-        if (need + tree.NumNodes() > freeNodes()) break;
-        need += (uint32_t)tree.NumNodes();
+        if (units[t] + 2 * tileUnits > groupCapacity)
+          throw Error("a tree of " + std::to_string(forest.trees[t].NumNodes()) + " nodes does not fit one LDS tree group");
+        if (need + units[t] > freeNodes()) break;
+        need += units[t];
         ++count;
       }
       if (count == 0) break; // group full
@@ -272,33 +635,12 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
           continue;
         }
         const int32_t t = order[next + k];
-        const Tree &tree = forest.trees[t];
-        const LevelOrder lo = MakeLevelOrder(tree);
-        const uint32_t base = (uint32_t)pm.nodes.size() - g.nodeBegin; // node index inside the group
+        const uint32_t base = (uint32_t)pm.nodes.size() - g.nodeBegin; // unit index inside the group
         b.root[k] = (uint16_t)(base * kNodeBytes);
         b.depth = std::max<uint32_t>(b.depth, (uint32_t)depth[t]);
+        b.peelDepth = std::max<uint32_t>(b.peelDepth, (uint32_t)peel[t]);
         pm.slotTree.push_back(t);
-        for (size_t i = 0; i < lo.order.size(); ++i) {
-          const int32_t n = lo.order[i];
-          DeviceNode dn;
-          dn.value = tree.value[n];
-          if (plan.quantizedRows && !tree.IsLeaf(n)) {
-            const auto &sorted = ranks[(size_t)tree.feature[n]];
-            const uint32_t j = (uint32_t)(std::lower_bound(sorted.begin(), sorted.end(), tree.value[n]) - sorted.begin());
-            static_assert(sizeof(float) == sizeof(uint32_t), "node value holds the rank bit pattern");
-            std::memcpy(&dn.value, &j, sizeof(j));
-          }
-          if (tree.IsLeaf(n)) {
-            dn.meta = (((base + (uint32_t)i) * kNodeBytes) << 16) | (uint32_t)padOffset;
-          } else {
-            const uint32_t child = base + (uint32_t)lo.position[tree.left[n]];
-            if (lo.position[tree.right[n]] != lo.position[tree.left[n]] + 1)
-              throw Error("internal error: siblings not adjacent");
-            dn.meta = ((child * kNodeBytes) << 16) | ((uint32_t)tree.feature[n] * featureStride);
-          }
-          pm.nodes.push_back(dn);
-          pm.nodeOrigin.push_back(n);
-        }
+        emitTree(t, base);
       }
       for (int k = 0; k < K; ++k) pm.bundleRoots.push_back(pm.nodes[g.nodeBegin + b.root[k] / kNodeBytes]);
       pm.bundles.push_back(b);
@@ -328,6 +670,7 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan) {
 }
 
 Tree UnpackTree(const PackedModel &pm, int32_t treeIndex) {
+  if (pm.plan.tileSize > 1) throw Error("tiled models are checked through their walks, not unpacked");
   if (pm.plan.kernel == LaunchPlan::Kernel::kGlobalWalk) {
     for (const DeviceGlobalTree &gt : pm.globalTrees) {
       if (gt.origin != treeIndex) continue;

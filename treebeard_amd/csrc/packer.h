@@ -33,6 +33,17 @@ struct LaunchPlan {
   // by the number of that feature's split thresholds that are <= it (one byte), which preserves the
   // outcome of every comparison; 64 rows of 1 byte per feature then fit LDS where 64 f32 rows do not.
   bool quantizedRows = false;
+  // Tiled walk (row-parallel kernel on f32 rows only): nodes per tile, 1 = scalar nodes.  How the members of a
+  // tile are chosen follows the reference: 0 breadth first (src/mlir/UniformTilingTransformation.cpp:148-195),
+  // 1 most-visited child first on trees whose profile is skewed, 2 the same but breadth first below nodes that
+  // fewer than 20 % of the rows reach (src/mlir/ProbabilityBasedTilingTransform.cpp:124-198, :243-262); 1 and
+  // 2 need a hit-count profile and fall back to 0 without one.
+  int32_t tileSize = 1;
+  int32_t tiling = 0;
+  // Walk peeling (src/mlir/ProbabilityBasedTilingTransform.cpp:66-73): with a profile, a bundle first takes the
+  // steps that bring 90 % of the profiled rows to their leaves without looking, then steps on only while some
+  // lane of the wave still moves.
+  bool peelWalks = false;
 
   int32_t ThreadsPerBlock() const {
     if (kernel == Kernel::kGlobalWalk) return rowsPerBlock;
@@ -61,6 +72,12 @@ struct PackedModel {
   // the f32 row-parallel walk takes level 0 from scalar registers instead of an LDS node read.
   std::vector<DeviceNode> bundleRoots;
   uint32_t maxGroupNodes = 0;
+  // Tiled plans: how many trees were tiled by visit counts (the others breadth first), and the tile steps
+  // one row takes over the whole forest: lock-step (deepest leaf of every tree) and, when a profile was
+  // given, what the profiled rows need on average.
+  int32_t treesTiledByProfile = 0;
+  int64_t lockStepSteps = 0;
+  double profiledSteps = 0.0;
   // kGlobalWalk only:
   std::vector<DeviceGlobalNode> globalNodes;
   std::vector<DeviceGlobalTree> globalTrees; // ordered by (class, depth)
@@ -89,8 +106,9 @@ struct PackedModel {
 int32_t MaxThresholdsPerFeature(const Forest &forest);
 
 // Throws tbamd::Error when the plan cannot hold the model (tree larger than a
-// group, feature offsets that do not fit 16 bits, ...).
-PackedModel PackForest(const Forest &forest, const LaunchPlan &plan);
+// group, feature offsets that do not fit 16 bits, ...).  `profile` (may be null) feeds the plan's
+// probability-based tiling and walk peeling.
+PackedModel PackForest(const Forest &forest, const LaunchPlan &plan, const HitCountProfile *profile = nullptr);
 
 // Inverse of PackForest for tests: rebuilds (value, feature, left, right) of
 // original tree `tree` from the packed arrays.

@@ -8,6 +8,7 @@ namespace tbamd {
 
 bool gMeasureGpuKernelTime = false;
 int32_t gNumberOfKernelRuns = 1;
+bool gPeeledWalks = false;
 
 namespace {
 
@@ -51,11 +52,14 @@ template <typename T> T *Upload(const std::vector<T> &host, const char *what) {
 } // namespace
 
 InferenceRunner::InferenceRunner(Forest forest, const CompilerOptions &options,
-                                 const GPUAutoScheduleOptions *gpuOptions)
-    : m_forest(std::move(forest)), m_options(options) {
+                                 const GPUAutoScheduleOptions *gpuOptions, std::unique_ptr<HitCountProfile> profile)
+    : m_forest(std::move(forest)), m_profile(std::move(profile)), m_options(options) {
   try {
     InitDevice();
-    m_model = PackForest(m_forest, ChoosePlan(m_forest, m_options.batchSize, gpuOptions, m_limits));
+    m_walk.tileSize = m_options.tileSize;
+    m_walk.tiling = m_profile ? (int32_t)m_options.tilingType : 0;
+    m_walk.peelWalks = m_profile && gPeeledWalks;
+    m_model = PackForest(m_forest, ChoosePlan(m_forest, m_options.batchSize, gpuOptions, m_limits, m_walk), m_profile.get());
     UploadModel();
   } catch (...) { // a constructor that throws gets no destructor call: give back what was created
     Release();
@@ -63,11 +67,16 @@ InferenceRunner::InferenceRunner(Forest forest, const CompilerOptions &options,
   }
 }
 
-InferenceRunner::InferenceRunner(Forest forest, const CompilerOptions &options, const LaunchPlan &plan)
-    : m_forest(std::move(forest)), m_options(options) {
+InferenceRunner::InferenceRunner(Forest forest, const CompilerOptions &options, const LaunchPlan &plan,
+                                 std::unique_ptr<HitCountProfile> profile)
+    : m_forest(std::move(forest)), m_profile(std::move(profile)), m_options(options) {
   try {
+    m_options.tileSize = plan.tileSize;
     InitDevice();
-    m_model = PackForest(m_forest, plan);
+    m_walk.tileSize = plan.tileSize;
+    m_walk.tiling = plan.tiling;
+    m_walk.peelWalks = plan.peelWalks;
+    m_model = PackForest(m_forest, plan, m_profile.get());
     UploadModel();
   } catch (...) {
     Release();
@@ -159,7 +168,7 @@ void InferenceRunner::UploadModel() {
 }
 
 void InferenceRunner::Repack(const LaunchPlan &plan) {
-  PackedModel next = PackForest(m_forest, plan);
+  PackedModel next = PackForest(m_forest, plan, m_profile.get());
   // refuse before anything is freed: a plan that fails leaves the runner as it was
   if (next.LdsBytes() > (size_t)m_limits.ldsBytesPerBlock) throw Error("launch plan exceeds the LDS of one workgroup");
   Check(hipStreamSynchronize(m_stream), "hipStreamSynchronize");
@@ -235,6 +244,7 @@ hipError_t InferenceRunner::LaunchWalk(const WalkParams &p, hipStream_t stream) 
   if (plan.kernel == LaunchPlan::Kernel::kGlobalWalk) return LaunchWalkGlobal(p, plan.interleave, stream);
   if (plan.kernel == LaunchPlan::Kernel::kTreeParallel)
     return LaunchWalkTreeParallel(p, plan.interleave, m_model.LdsBytes(), stream);
+  if (plan.tileSize > 1) return LaunchWalkRowsTiled(p, plan.tileSize, plan.interleave, m_model.LdsBytes(), stream);
   const int tileMode = plan.quantizedRows ? 2 : (plan.featureOffsetInWords ? 1 : 0);
   return LaunchWalkRowsLds(p, plan.interleave, tileMode, m_model.LdsBytes(), stream);
 }
@@ -512,7 +522,7 @@ double InferenceRunner::AutoTune(const float *deviceInputs, int64_t rows) {
   LaunchPlan best = original;
   double bestMs = 1e300;
   try {
-    for (const LaunchPlan &cand : CandidatePlans(m_forest, rows, m_limits)) {
+    for (const LaunchPlan &cand : CandidatePlans(m_forest, rows, m_limits, m_walk)) {
       try {
         Repack(cand);
       } catch (const Error &) {
@@ -553,7 +563,9 @@ std::string InferenceRunner::DescribePlan() const {
      << " offsetsInWords=" << (p.featureOffsetInWords ? 1 : 0) << " quantizedRows=" << (p.quantizedRows ? 1 : 0)
      << " groups=" << m_model.groups.size()
      << " bundles=" << m_model.bundles.size() << " nodes=" << m_model.nodes.size()
-     << " ldsBytes=" << m_model.LdsBytes();
+     << " ldsBytes=" << m_model.LdsBytes() << " tileSize=" << p.tileSize << " tiling=" << p.tiling
+     << " peelWalks=" << (p.peelWalks ? 1 : 0) << " treesTiledByProfile=" << m_model.treesTiledByProfile
+     << " lockStepSteps=" << m_model.lockStepSteps << " profiledSteps=" << m_model.profiledSteps;
   return os.str();
 }
 

@@ -25,12 +25,19 @@ namespace tbamd {
 // (src/gpu/GPUSupportUtils.cpp:52-104, :389-390).
 extern bool gMeasureGpuKernelTime;
 extern int32_t gNumberOfKernelRuns;
+// The reference's switch for peeled walks under probability-based tiling
+// (SetPeeledCodeGenForProbabilityBasedTiling, src/runtime/runtime.cpp:309-315); read when a runner is made.
+extern bool gPeeledWalks;
 
 class InferenceRunner {
 public:
-  InferenceRunner(Forest forest, const CompilerOptions &options, const GPUAutoScheduleOptions *gpuOptions);
+  // `profile` (may be null): leaf hit counts for probability-based tiling and walk peeling, used when the
+  // options ask for a non-uniform tiling type.
+  InferenceRunner(Forest forest, const CompilerOptions &options, const GPUAutoScheduleOptions *gpuOptions,
+                  std::unique_ptr<HitCountProfile> profile = nullptr);
   // Reopens a compiled model: the plan is taken as saved instead of asking the tuner.
-  InferenceRunner(Forest forest, const CompilerOptions &options, const LaunchPlan &plan);
+  InferenceRunner(Forest forest, const CompilerOptions &options, const LaunchPlan &plan,
+                  std::unique_ptr<HitCountProfile> profile = nullptr);
   ~InferenceRunner();
   InferenceRunner(const InferenceRunner &) = delete;
   InferenceRunner &operator=(const InferenceRunner &) = delete;
@@ -77,6 +84,7 @@ public:
   int64_t LastKernelMicros() const { return m_lastKernelMicros; }
   const PackedModel &Model() const { return m_model; }
   const Forest &GetForest() const { return m_forest; }
+  const HitCountProfile *Profile() const { return m_profile.get(); }
   std::string DescribePlan() const;
   hipStream_t Stream() const { return m_stream; }
 
@@ -107,6 +115,8 @@ private:
               float *probabilities, int32_t *leafIds, hipStream_t stream, const Workspace &ws);
 
   Forest m_forest;
+  std::unique_ptr<HitCountProfile> m_profile;
+  WalkOptions m_walk;
   CompilerOptions m_options;
   DeviceLimits m_limits;
   PackedModel m_model;

@@ -74,9 +74,18 @@ Forest LoadByType(const std::string &path, const std::string &type, int32_t numF
   throw Error("unknown forest creator type " + type);
 }
 
+// The leaf hit-count profile the options name, when they ask for a tiling type that uses one
+// (src/mlir/ProbabilityBasedTilingTransform.cpp:124-198 reads the same counts from the model's nodes).
+std::unique_ptr<HitCountProfile> ProfileFor(const Forest &forest, const CompilerOptions &options) {
+  if (options.statsProfileCSVPath.empty() || options.tilingType == TilingType::kUniform) return nullptr;
+  return std::make_unique<HitCountProfile>(LoadHitCountProfile(forest, options.statsProfileCSVPath));
+}
+
 InferenceRunner *RunnerFromContext(Context *ctx) {
   Forest forest = ctx->forest ? *ctx->forest : LoadByType(ctx->modelPath, ctx->creatorType, ctx->options.numberOfFeatures);
-  return new InferenceRunner(std::move(forest), ctx->options, ctx->hasGpuOptions ? &ctx->gpuOptions : nullptr);
+  std::unique_ptr<HitCountProfile> profile = ProfileFor(forest, ctx->options);
+  return new InferenceRunner(std::move(forest), ctx->options, ctx->hasGpuOptions ? &ctx->gpuOptions : nullptr,
+                             std::move(profile));
 }
 
 // Rows for the timed plan search: `<model>.test.sampled.csv` next to the model
@@ -187,11 +196,8 @@ intptr_t CreateInferenceRunner(const char *modelJSONPath, const char *profileCSV
         CompilerOptions opts = *Opts(options);
         if (profileCSVPath && *profileCSVPath) opts.statsProfileCSVPath = profileCSVPath;
         Forest forest = LoadXGBoostJSON(modelJSONPath);
-        // A hit-count profile is checked against the model; the lock-step kernels have no
-        // data-dependent layout, so it does not change the packed model.
-        if (!opts.statsProfileCSVPath.empty() && opts.tilingType != TilingType::kUniform)
-          (void)LoadHitCountProfile(forest, opts.statsProfileCSVPath);
-        return reinterpret_cast<intptr_t>(new InferenceRunner(std::move(forest), opts, nullptr));
+        std::unique_ptr<HitCountProfile> profile = ProfileFor(forest, opts);
+        return reinterpret_cast<intptr_t>(new InferenceRunner(std::move(forest), opts, nullptr, std::move(profile)));
       },
       0);
 }
@@ -200,8 +206,9 @@ intptr_t CreateInferenceRunnerForONNXModel(const char *modelPath, intptr_t optio
   return Guard(
       [&]() -> intptr_t {
         CompilerOptions opts = *Opts(options);
-        return reinterpret_cast<intptr_t>(
-            new InferenceRunner(LoadONNX(modelPath, opts.numberOfFeatures), opts, nullptr));
+        Forest forest = LoadONNX(modelPath, opts.numberOfFeatures);
+        std::unique_ptr<HitCountProfile> profile = ProfileFor(forest, opts);
+        return reinterpret_cast<intptr_t>(new InferenceRunner(std::move(forest), opts, nullptr, std::move(profile)));
       },
       0);
 }
@@ -209,7 +216,10 @@ intptr_t CreateInferenceRunnerForONNXModel(const char *modelPath, intptr_t optio
 // ---- process-wide switches ----
 void SetEnableSparseRepresentation(int32_t val) { gSparseRepresentation = val; }
 int32_t IsSparseRepresentationEnabled(void) { return gSparseRepresentation; }
-void SetPeeledCodeGenForProbabilityBasedTiling(int32_t val) { gPeeledCodeGen = val; }
+void SetPeeledCodeGenForProbabilityBasedTiling(int32_t val) {
+  gPeeledCodeGen = val;
+  gPeeledWalks = val != 0;
+}
 int32_t IsPeeledCodeGenForProbabilityBasedTilingEnabled(void) { return gPeeledCodeGen; }
 void SetEnableMeasureGpuKernelTime(bool val) { gMeasureGpuKernelTime = val; }
 void SetNumberOfKernelRuns(int32_t val) { gNumberOfKernelRuns = val < 1 ? 1 : val; }
@@ -469,7 +479,7 @@ int32_t tbmi_save_compiled_model(intptr_t h, const char *path) {
       [&] {
         InferenceRunner *r = Runner(h);
         SaveCompiledModel(path ? path : "", r->GetForest(), r->Model().plan, r->BatchSize(),
-                          r->Options().returnTypeWidth, r->Options().returnTypeFloatType);
+                          r->Options().returnTypeWidth, r->Options().returnTypeFloatType, r->Profile());
         return 0;
       },
       -1);
@@ -483,7 +493,7 @@ intptr_t tbmi_load_compiled_model(const char *path, int32_t batchSize) {
         options.batchSize = batchSize > 0 ? batchSize : m.batchSize;
         options.returnTypeWidth = m.returnTypeWidth;
         options.returnTypeFloatType = m.returnTypeFloatType;
-        return reinterpret_cast<intptr_t>(new InferenceRunner(std::move(m.forest), options, m.plan));
+        return reinterpret_cast<intptr_t>(new InferenceRunner(std::move(m.forest), options, m.plan, std::move(m.profile)));
       },
       0);
 }

@@ -76,8 +76,64 @@ LaunchPlan ChooseTreeParallelPlan(const Forest &forest, int64_t batchSize, const
 
 } // namespace
 
+namespace {
+LaunchPlan ChooseScalarPlan(const Forest &forest, int64_t batchSize, const GPUAutoScheduleOptions *ov,
+                            const DeviceLimits &limits, bool tiled);
+}
+
 LaunchPlan ChoosePlan(const Forest &forest, int64_t batchSize, const GPUAutoScheduleOptions *ov,
-                      const DeviceLimits &limits) {
+                      const DeviceLimits &limits, const WalkOptions &walk) {
+  if (walk.tileSize < 1 || walk.tileSize > kMaxTileSize)
+    throw Error("tile size " + std::to_string(walk.tileSize) + " is not supported: the device kernels walk tiles of 1 to " +
+                std::to_string(kMaxTileSize) + " nodes");
+  LaunchPlan plan = ChooseScalarPlan(forest, batchSize, ov, limits, walk.tileSize > 1);
+  plan.tileSize = walk.tileSize;
+  plan.tiling = walk.tiling;
+  plan.peelWalks = walk.peelWalks;
+  return plan;
+}
+
+namespace {
+
+// `tiled`: the plan must be the row-parallel kernel on f32 rows with byte offsets (tiles hold byte offsets
+// into a row tile below 64 KB), and groups are sized for tiles, which take about three times the bytes of
+// scalar nodes.
+LaunchPlan ChooseScalarPlan(const Forest &forest, int64_t batchSize, const GPUAutoScheduleOptions *ov,
+                            const DeviceLimits &limits, bool tiled) {
+  if (tiled) {
+    if ((BiggestTreeNodes(forest) + 2) * 32 > 65536)
+      throw Error("tile sizes above 1 need every tree to fit one LDS tree group; this forest has a tree that does not");
+    LaunchPlan plan;
+    plan.kernel = LaunchPlan::Kernel::kRowParallelLds;
+    int32_t rb = 256;
+    if (ov && ov->numRowsPerTB > 0) rb = std::max(64, std::min(256, FloorPow2(ov->numRowsPerTB)));
+    // two blocks per CU while 24 KB remain for a group, byte offsets below 64 KB
+    auto tileBytes = [&](int32_t r) { return (int64_t)(forest.numFeatures + 1) * r * 4; };
+    while (rb > 64 && (tileBytes(rb) > 0xFFFF || limits.ldsBytesPerBlock / 2 - tileBytes(rb) < 24 * 1024)) rb /= 2;
+    if (tileBytes(rb) > 0xFFFF)
+      throw Error("tile sizes above 1 need a row tile below 64 KB: " + std::to_string(forest.numFeatures) + " features are too many");
+    plan.rowsPerBlock = rb;
+    plan.treeThreads = std::max(1, 1024 / rb);
+    if (ov && ov->numTreeThreads > 0) plan.treeThreads = std::max(1, std::min(ov->numTreeThreads, 1024 / rb));
+    plan.interleave = 2;
+    if (ov && ov->treeWalkInterleaveFactor > 0) plan.interleave = std::min(4, FloorPow2(ov->treeWalkInterleaveFactor));
+    const int64_t meet = forest.numClasses > 0 ? (int64_t)rb * plan.treeThreads * 8 : 0;
+    int64_t budget = limits.ldsBytesPerBlock / 2;
+    int64_t group = std::min<int64_t>(65536, budget - tileBytes(rb) - meet - 512);
+    const int64_t need = (BiggestTreeNodes(forest) + 2) * 32;
+    if (group < need) group = std::min<int64_t>(65536, limits.ldsBytesPerBlock - tileBytes(rb) - meet - 512);
+    group = std::min<int64_t>(group, 256LL * rb * plan.treeThreads);
+    if (group < need) throw Error("the biggest tree does not fit LDS next to the row tile when tiled");
+    plan.groupBytes = (int32_t)(group & ~15);
+    const int64_t rowBlocks = std::max<int64_t>(1, (batchSize + rb - 1) / rb);
+    const int64_t totalBytes = (int64_t)forest.NumNodes() * 24;
+    int64_t slices = 1;
+    const int64_t wantBlocks = 2LL * limits.computeUnits;
+    if (rowBlocks < wantBlocks) slices = (wantBlocks + rowBlocks - 1) / rowBlocks;
+    slices = std::min<int64_t>(slices, std::max<int64_t>(1, totalBytes / plan.groupBytes));
+    plan.treeSlices = (int32_t)std::max<int64_t>(1, slices);
+    return plan;
+  }
   if ((BiggestTreeNodes(forest) + 2) * kNodeBytes > 65536) {
     // A tree that cannot sit in one LDS group: walk from global memory.
     LaunchPlan plan;
@@ -206,10 +262,34 @@ LaunchPlan ChoosePlan(const Forest &forest, int64_t batchSize, const GPUAutoSche
   return plan;
 }
 
-std::vector<LaunchPlan> CandidatePlans(const Forest &forest, int64_t batchSize, const DeviceLimits &limits) {
+} // namespace
+
+std::vector<LaunchPlan> CandidatePlans(const Forest &forest, int64_t batchSize, const DeviceLimits &limits,
+                                       const WalkOptions &walk) {
   std::vector<LaunchPlan> out;
-  LaunchPlan base = ChoosePlan(forest, batchSize, nullptr, limits);
+  LaunchPlan base = ChoosePlan(forest, batchSize, nullptr, limits, walk);
   out.push_back(base);
+  if (base.tileSize > 1) { // block shapes and interleave factors of the tiled walk
+    for (int32_t rb : {64, 128, 256})
+      for (int32_t k : {1, 2, 4}) {
+        LaunchPlan p = base;
+        p.rowsPerBlock = rb;
+        p.treeThreads = 1024 / rb;
+        p.interleave = k;
+        const int64_t tile = (int64_t)(forest.numFeatures + 1) * rb * 4;
+        if (tile > 0xFFFF) continue;
+        const int64_t meet = forest.numClasses > 0 ? (int64_t)rb * p.treeThreads * 8 : 0;
+        int64_t group = std::min<int64_t>(65536, limits.ldsBytesPerBlock / 2 - tile - meet - 2048);
+        if (group < (BiggestTreeNodes(forest) + 2) * 32) continue;
+        if (base.treeSlices > 1) group = std::min<int64_t>(group, base.groupBytes);
+        p.groupBytes = (int32_t)(group & ~15);
+        bool dup = false;
+        for (auto &q : out)
+          dup = dup || (q.rowsPerBlock == p.rowsPerBlock && q.interleave == p.interleave && q.groupBytes == p.groupBytes);
+        if (!dup) out.push_back(p);
+      }
+    return out;
+  }
   if (base.kernel == LaunchPlan::Kernel::kGlobalWalk) {
     for (int32_t k : {1, 2, 8}) {
       LaunchPlan p = base;

@@ -17,11 +17,21 @@ struct DeviceLimits {
   int32_t ldsBytesPerBlock = 160 * 1024;
 };
 
-// Analytic choice; `overrides` (may be null) pins what the caller set.
+// What the compiler options ask of the walk itself (CompilerOptions::tileSize, tilingType and the peeled
+// code generation switch); copied into the plan.
+struct WalkOptions {
+  int32_t tileSize = 1;
+  int32_t tiling = 0;     // 0 uniform, 1 probabilistic, 2 hybrid
+  bool peelWalks = false;
+};
+
+// Analytic choice; `overrides` (may be null) pins what the caller set.  Tile sizes above 1 always get the
+// row-parallel kernel on f32 rows (the only one that walks tiles) and fail when its row tile does not fit.
 LaunchPlan ChoosePlan(const Forest &forest, int64_t batchSize, const GPUAutoScheduleOptions *overrides,
-                      const DeviceLimits &limits);
+                      const DeviceLimits &limits, const WalkOptions &walk = WalkOptions());
 
 // Candidate plans for the timed search (the analytic choice comes first).
-std::vector<LaunchPlan> CandidatePlans(const Forest &forest, int64_t batchSize, const DeviceLimits &limits);
+std::vector<LaunchPlan> CandidatePlans(const Forest &forest, int64_t batchSize, const DeviceLimits &limits,
+                                       const WalkOptions &walk = WalkOptions());
 
 } // namespace tbamd
