@@ -191,6 +191,18 @@ void WalkRowLds(const WalkParams &p, int K, uint32_t stride, bool rankRows, int6
 
 void StoreRow(const WalkParams &p, int64_t row, int slice, const double *classSums) {
   const int C = p.s.numClasses;
+  if (p.s.fuseArgmax) { // the kernel's own running arg-max (ties go to the larger class id)
+    if (C <= 0 || p.s.treeSlices != 1 || p.partial || (!p.out && !p.classOut)) std::abort();
+    float best = -INFINITY;
+    int bestClass = 0;
+    for (int c = 0; c < C; ++c) {
+      const float m = (float)(p.s.initialValue + classSums[c]);
+      if (!(best > m)) best = m, bestClass = c;
+    }
+    if (p.classOut) p.classOut[row] = (int8_t)bestClass;
+    else p.out[row] = (float)bestClass;
+    return;
+  }
   if (C > 0 || p.partial) {
     if (!p.partial) std::abort(); // classifiers always go through the finalize kernel
     double *dst = p.partial + ((int64_t)slice * p.s.rows + row) * (C > 0 ? C : 1);

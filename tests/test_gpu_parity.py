@@ -515,7 +515,7 @@ def test_global_walk_plans_agree(synth_model, k, plan):
     check_against_oracle(runner, forest, x)
 
 
-@pytest.mark.parametrize("kernel", ["rows_lds", "tree_parallel", "global_walk"])
+@pytest.mark.parametrize("kernel", ["rows_lds", "rows_lds_one_slice", "tree_parallel", "global_walk"])
 def test_classes_without_trees_score_the_initial_value(tmp_path, kernel):
     """The reference's two sides disagree on a class no tree votes for: its generated code fills every class
     sum with the initial value before reducing (src/reduction/LowerReduceOps.cpp:1459-1470,
@@ -533,11 +533,13 @@ def test_classes_without_trees_score_the_initial_value(tmp_path, kernel):
     runner = make_runner(path, rows)
     if kernel == "rows_lds":
         runner.set_plan(64, 2, 2, 4096, 3)
+    elif kernel == "rows_lds_one_slice":
+        runner.set_plan(64, 2, 2, 4096, 1)      # one tree slice: the walk kernel keeps the arg-max itself
     elif kernel == "tree_parallel":
         runner.set_tree_parallel_plan(4, 16, 2, 0, 2)
     else:
         runner.set_global_walk_plan(128, 2, 4)
-    assert "kernel=" + kernel in runner.describe_plan()
+    assert "kernel=" + kernel.replace("_one_slice", "") in runner.describe_plan()
     np.testing.assert_array_equal(gpu_leaf_ids(runner, x), cpu_oracle.leaf_ids(forest, x))
     _, sums = cpu_oracle.predict(forest, x)
     voted = np.isin(np.arange(7), info)
@@ -549,6 +551,36 @@ def test_classes_without_trees_score_the_initial_value(tmp_path, kernel):
     runner.run_device_multiclass(dx.data_ptr(), rows, classes.data_ptr(), margins.data_ptr(), None)
     np.testing.assert_allclose(margins.cpu().numpy(), expected, rtol=RTOL_SUM, atol=1e-7)
     np.testing.assert_array_equal(classes.cpu().numpy(), cpu_oracle.argmax_generated(expected))
+    np.testing.assert_array_equal(gpu_predict(runner, x), cpu_oracle.argmax_generated(expected))   # class ids only
+
+
+@pytest.mark.parametrize("slices,tile_size", [(1, 1), (3, 1), (1, 2), (1, 4)])
+def test_class_ties_go_to_the_larger_class_id(tmp_path, slices, tile_size):
+    """Exact ties between class sums: the generated code replaces the running maximum unless it is strictly
+    greater (src/reduction/LowerReduceOps.cpp:148-187), so the larger class id wins - in the finalize kernel
+    and in the walk kernels' own arg-max (one tree slice)."""
+    rng = np.random.Generator(np.random.PCG64(21))
+    split = lambda: (rng.integers(0, 4), rng.normal())
+    base = [synth._grow_tree(rng, 3, lambda d, s: 0.9, split, lambda: float(rng.integers(-2, 3)) * 0.25) for _ in range(6)]
+    trees, info = [], []
+    for c in (1, 3, 4):                  # three classes get the same trees: their sums tie on every row
+        trees += base
+        info += [c] * len(base)
+    trees.append(base[0]); info.append(0)
+    path = tmp_path / "ties.json"
+    synth.write_xgboost_json(path, trees, 4, objective="multi:softmax", num_class=6, tree_info=info)
+    forest = model_io.load_xgboost_json(path)
+    rows = 900
+    x = rng.normal(size=(rows, 4)).astype(np.float32)
+    runner = make_tiled_runner(path, rows, tile_size, multiclass=True)
+    runner.set_plan(64, 2, 2, 4096, slices)
+    _, sums = cpu_oracle.predict(forest, x)
+    voted = np.isin(np.arange(6), info)
+    margins = np.where(voted[None, :], sums, forest.initial_value).astype(np.float32)
+    expected = cpu_oracle.argmax_generated(margins)
+    assert (margins[:, 1] == margins[:, 3]).all() and (margins[:, 3] == margins[:, 4]).all()
+    assert set(np.unique(expected)) >= {4}            # the tie is the maximum on some rows and then class 4 wins
+    np.testing.assert_array_equal(gpu_predict(runner, x), expected)
 
 
 @pytest.mark.parametrize("fine", [False, True], ids=["coarse_thresholds", "fine_thresholds"])

@@ -36,7 +36,8 @@ def _both(runner, x):
 
 # (configuration, plan, rows of the first call, rows of the second call)
 CASES = [
-    (3, None, 6000, 1111),                       # classifier: per-class partial sums + finalize
+    (3, None, 6000, 1111),                       # classifier, one tree slice: arg-max kept by the walk kernel
+    (3, ("plan", 256, 4, 4, 0, 2), 6000, 1111),  # classifier over two tree slices: per-class partial sums + finalize
     (2, ("plan", 256, 4, 4, 16384, 6), 3000, 500),   # tree slices: partial sums per slice
     (2, None, 70000, 4097),                      # fused epilogue: no scratch memory at all
     (4, None, 1024, 300),                        # rank-quantised rows (+ tree slices at this size)
@@ -60,8 +61,9 @@ def test_no_alloc_entry_point_matches_run_device(synth_model, k, plan, first, se
 def test_no_alloc_entry_point_rejects_what_does_not_fit(synth_model):
     limit = api().runtime_lib.tbmi_noalloc_scratch_bytes()
     assert limit == 32 << 20
-    rows = limit // (8 * 8) + 1                  # configuration 3: 8 classes x 8 bytes of partial sums per row
-    runner = _runner(synth_model(3), rows, True)               # a batch this size gets a plan without tree slices
+    rows = limit // (2 * 8 * 8) + 1              # configuration 3 over two tree slices: 2 x 8 classes x 8 bytes per row
+    runner = _runner(synth_model(3), rows, True)
+    runner.set_plan(256, 4, 4, 0, 2)             # (with one slice the walk keeps the arg-max itself and needs no scratch)
     dx = torch.zeros((rows, 54), dtype=torch.float32, device="cuda")
     out = torch.zeros((rows,), dtype=torch.int8, device="cuda")
     torch.cuda.synchronize()

@@ -20,6 +20,9 @@ struct WalkScalars {
   int32_t rowsPerBlock = 0;      // rows per block (both kernels)
   int32_t treeThreads = 1;       // row-parallel kernel: lanes (in different waves) that share a row
   int32_t treeLanes = 1;         // tree-parallel kernel: lanes per row (power of two)
+  // Row-parallel kernels, classifiers with one tree slice: the kernel keeps the running arg-max of the class
+  // sums (which arrive in ascending class order) and stores the class id itself; no partial sums, no finalize.
+  int32_t fuseArgmax = 0;
   double initialValue = 0.0;
 };
 
@@ -32,7 +35,8 @@ struct WalkParams {
   const DeviceGroup *groups = nullptr;
   const DeviceGlobalNode *globalNodes = nullptr; // global-memory walk only
   const DeviceGlobalTree *globalTrees = nullptr;
-  float *out = nullptr;           // used when the epilogue is fused (1 slice, no classes)
+  float *out = nullptr;           // used when the epilogue is fused (1 slice; class ids as float32 with fuseArgmax)
+  int8_t *classOut = nullptr;     // fuseArgmax: class ids as int8 (out is then null)
   double *partial = nullptr;      // [partials][rows][max(1, classes)] otherwise
   // leaf-id dump (parity checks only)
   int32_t *leafIds = nullptr;     // [rows][numTrees]

@@ -119,8 +119,8 @@ __global__ void __launch_bounds__(1024)
 WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16,
                   const DeviceBundle *__restrict__ bundles, const DeviceNode *__restrict__ bundleRoots,
                   const DeviceGroup *__restrict__ groups,
-                  const WalkScalars s, float *__restrict__ out, double *__restrict__ partial,
-                  int32_t *__restrict__ leafIds, const int32_t *__restrict__ nodeOrigin,
+                  const WalkScalars s, float *__restrict__ out, int8_t *__restrict__ classOut,
+                  double *__restrict__ partial, int32_t *__restrict__ leafIds, const int32_t *__restrict__ nodeOrigin,
                   const int32_t *__restrict__ slotTree) {
   // LDS: [tree group nodes | transposed row tile].  The group sits at LDS
   // address 0 so that node pointers are LDS addresses as stored.
@@ -181,6 +181,8 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
 
   double acc = 0.0;
   int curClass = 0;
+  float best = -INFINITY; // fuseArgmax: running maximum of the class sums and its class (tree thread 0)
+  int bestClass = 0;
 
   // Register double buffer for the next tree group.  Loads are unconditional
   // (index clamped) so that they stay in flight across the walk.
@@ -208,7 +210,15 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
         for (int t = 0; t < TT; ++t) acc += meet[t * RB + lane];                                                       \
       }                                                                                                                \
     }                                                                                                                  \
-    if (tt == 0 && lane < valid) {                                                                                     \
+    if (s.fuseArgmax) {                                                                                                \
+      /* running arg-max with the generated code's tie rule (replace unless strictly greater); a class */              \
+      /* without trees scores the initial value */                                                                     \
+      const float m = (float)(s.initialValue + acc);                                                                   \
+      if (!(best > m)) { best = m; bestClass = curClass; }                                                             \
+      const float m0 = (float)s.initialValue;                                                                          \
+      for (int c = curClass + 1; c < (UPTO); ++c)                                                                      \
+        if (!(best > m0)) { best = m0; bestClass = c; }                                                                \
+    } else if (tt == 0 && lane < valid) {                                                                              \
       partialRow[curClass] = acc;                                                                                      \
       for (int c = curClass + 1; c < (UPTO); ++c) partialRow[c] = 0.0;                                                 \
     }                                                                                                                  \
@@ -314,6 +324,10 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
 
   if (C > 0) {
     TBAMD_FLUSH_CLASS(C)
+    if (s.fuseArgmax && tt == 0 && lane < valid) {
+      if (classOut) classOut[row] = (int8_t)bestClass;
+      else out[row] = (float)bestClass;
+    }
     return;
   }
   if (TT > 1) {
@@ -392,8 +406,8 @@ template <int T, int K, int PF, bool kDump>
 __global__ void __launch_bounds__(1024)
 WalkRowsTiledKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16,
                     const DeviceBundle *__restrict__ bundles, const DeviceGroup *__restrict__ groups,
-                    const WalkScalars s, float *__restrict__ out, double *__restrict__ partial,
-                    int32_t *__restrict__ leafIds, const int32_t *__restrict__ nodeOrigin,
+                    const WalkScalars s, float *__restrict__ out, int8_t *__restrict__ classOut,
+                    double *__restrict__ partial, int32_t *__restrict__ leafIds, const int32_t *__restrict__ nodeOrigin,
                     const int32_t *__restrict__ slotTree) {
   extern __shared__ __align__(16) unsigned char lds[];
   const int tid = threadIdx.x;
@@ -422,6 +436,8 @@ WalkRowsTiledKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes
 
   double acc = 0.0;
   int curClass = 0;
+  float best = -INFINITY; // fuseArgmax: running maximum of the class sums and its class (tree thread 0)
+  int bestClass = 0;
   U32x4 fetched[PF];
 #define TBAMD_PREFETCH_GROUP(NEXTGRP)                                                                                  \
   {                                                                                                                    \
@@ -444,7 +460,15 @@ WalkRowsTiledKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes
         for (int t = 0; t < TT; ++t) acc += meet[t * RB + lane];                                                       \
       }                                                                                                                \
     }                                                                                                                  \
-    if (tt == 0 && lane < valid) {                                                                                     \
+    if (s.fuseArgmax) {                                                                                                \
+      /* running arg-max with the generated code's tie rule (replace unless strictly greater); a class */              \
+      /* without trees scores the initial value */                                                                     \
+      const float m = (float)(s.initialValue + acc);                                                                   \
+      if (!(best > m)) { best = m; bestClass = curClass; }                                                             \
+      const float m0 = (float)s.initialValue;                                                                          \
+      for (int c = curClass + 1; c < (UPTO); ++c)                                                                      \
+        if (!(best > m0)) { best = m0; bestClass = c; }                                                                \
+    } else if (tt == 0 && lane < valid) {                                                                              \
       partialRow[curClass] = acc;                                                                                      \
       for (int c = curClass + 1; c < (UPTO); ++c) partialRow[c] = 0.0;                                                 \
     }                                                                                                                  \
@@ -520,6 +544,10 @@ WalkRowsTiledKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes
 
   if (C > 0) {
     TBAMD_FLUSH_CLASS(C)
+    if (s.fuseArgmax && tt == 0 && lane < valid) {
+      if (classOut) classOut[row] = (int8_t)bestClass;
+      else out[row] = (float)bestClass;
+    }
     return;
   }
   if (TT > 1) {
@@ -972,12 +1000,12 @@ hipError_t LaunchWalkKP(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBy
     hipError_t e = AllowFullLds<&WalkRowsLdsKernel<K, PF, W, true>>();
     if (e != hipSuccess) return e;
     WalkRowsLdsKernel<K, PF, W, true><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.bundleRoots, p.groups, p.s, p.out,
-                                                                         p.partial, p.leafIds, p.nodeOrigin, p.slotTree);
+                                                                         p.classOut, p.partial, p.leafIds, p.nodeOrigin, p.slotTree);
   } else {
     hipError_t e = AllowFullLds<&WalkRowsLdsKernel<K, PF, W, false>>();
     if (e != hipSuccess) return e;
     WalkRowsLdsKernel<K, PF, W, false><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.bundleRoots, p.groups, p.s, p.out,
-                                                                          p.partial, nullptr, nullptr, nullptr);
+                                                                          p.classOut, p.partial, nullptr, nullptr, nullptr);
   }
   return hipGetLastError();
 }
@@ -1004,8 +1032,19 @@ hipError_t LaunchWalkW(const WalkParams &p, int interleave, int prefetch, dim3 g
 
 } // namespace
 
+namespace {
+// Outputs the walk kernels dereference must be there: a fused epilogue writes p.out (or p.classOut), everything
+// else goes through p.partial.
+bool OutputsConsistent(const WalkParams &p) {
+  if (p.s.fuseArgmax) return p.s.numClasses > 0 && p.s.treeSlices == 1 && (p.out || p.classOut);
+  if (p.s.numClasses > 0 || p.s.treeSlices > 1) return p.partial != nullptr;
+  return p.out != nullptr || p.partial != nullptr;
+}
+} // namespace
+
 hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, int tileMode, size_t ldsBytes, hipStream_t stream) {
   if (p.s.rows <= 0) return hipSuccess;
+  if (!OutputsConsistent(p)) return hipErrorInvalidValue;
   const int RB = p.s.rowsPerBlock, TT = p.s.treeThreads;
   if (ldsBytes > 160 * 1024 || RB < 64 || (RB & (RB - 1)) || TT < 1 || RB * TT > 1024) return hipErrorInvalidValue;
   const int64_t blocks = (p.s.rows + RB - 1) / RB;
@@ -1029,13 +1068,13 @@ hipError_t LaunchTiledTKP(const WalkParams &p, dim3 grid, dim3 block, size_t lds
   if (p.leafIds) {
     hipError_t e = AllowFullLds<&WalkRowsTiledKernel<T, K, PF, true>>();
     if (e != hipSuccess) return e;
-    WalkRowsTiledKernel<T, K, PF, true><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out, p.partial,
-                                                                          p.leafIds, p.nodeOrigin, p.slotTree);
+    WalkRowsTiledKernel<T, K, PF, true><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out, p.classOut,
+                                                                          p.partial, p.leafIds, p.nodeOrigin, p.slotTree);
   } else {
     hipError_t e = AllowFullLds<&WalkRowsTiledKernel<T, K, PF, false>>();
     if (e != hipSuccess) return e;
-    WalkRowsTiledKernel<T, K, PF, false><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out, p.partial,
-                                                                           nullptr, nullptr, nullptr);
+    WalkRowsTiledKernel<T, K, PF, false><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out, p.classOut,
+                                                                           p.partial, nullptr, nullptr, nullptr);
   }
   return hipGetLastError();
 }
@@ -1062,6 +1101,7 @@ hipError_t LaunchTiledT(const WalkParams &p, int interleave, int prefetch, dim3 
 
 hipError_t LaunchWalkRowsTiled(const WalkParams &p, int tileSize, int interleave, size_t ldsBytes, hipStream_t stream) {
   if (p.s.rows <= 0) return hipSuccess;
+  if (!OutputsConsistent(p)) return hipErrorInvalidValue;
   const int RB = p.s.rowsPerBlock, TT = p.s.treeThreads;
   if (ldsBytes > 160 * 1024 || RB < 64 || (RB & (RB - 1)) || TT < 1 || RB * TT > 1024) return hipErrorInvalidValue;
   // feature offsets are byte offsets into the f32 row tile: the tile has to end below 64 KB

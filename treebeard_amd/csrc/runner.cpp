@@ -277,8 +277,13 @@ void InferenceRunner::Launch(const float *deviceInputs, int64_t rows, float *out
                              float *probabilities, int32_t *leafIds, hipStream_t stream, const Workspace &ws) {
   if (rows <= 0) return;
   WalkParams p = MakeWalkParams(PrepareRows(deviceInputs, rows, ws.ranks, stream), rows);
-  const bool finalize = NeedsFinalize();
+  // A classifier whose trees all sit in one slice needs no second kernel when only the class id is wanted:
+  // the row-parallel kernels keep the running arg-max themselves.
+  const bool fused = FusesArgmax() && !margins && !probabilities;
+  const bool finalize = NeedsFinalize() && !fused;
+  p.s.fuseArgmax = fused ? 1 : 0;
   p.out = finalize ? nullptr : out;
+  p.classOut = fused ? classOut : nullptr;
   p.partial = finalize ? ws.partial : nullptr;
   if (leafIds) {
     p.leafIds = leafIds;
@@ -339,7 +344,7 @@ void InferenceRunner::RunDeviceNoAlloc(const float *deviceInputs, void *deviceRe
   if (rows < 0) throw Error("negative row count");
   if (rows == 0) return;
   if (!deviceInputs || !deviceResults) throw Error("null device buffer");
-  const size_t partialBytes = (PartialBytes(rows) + 255) & ~(size_t)255;
+  const size_t partialBytes = FusesArgmax() ? 0 : (PartialBytes(rows) + 255) & ~(size_t)255; // (no partial sums when the walk keeps the arg-max)
   const size_t ranksBytes = RanksBytes(rows);
   if (partialBytes + ranksBytes > kNoAllocScratchBytes)
     throw Error("this launch plan needs " + std::to_string(partialBytes + ranksBytes) + " bytes of scratch memory for " +
@@ -474,7 +479,8 @@ void InferenceRunner::TimeKernels(const float *deviceInputs, void *deviceResults
                                   double *walkMs, double *finalizeMs, double *binMs) {
   runs = std::max(1, runs);
   const Workspace ws = OwnWorkspace(rows);
-  const bool finalize = NeedsFinalize();
+  const bool fused = FusesArgmax();
+  const bool finalize = NeedsFinalize() && !fused;
   float ms = 0.f;
   if (binMs) *binMs = 0.0;
   const float *walkInputs = deviceInputs;
@@ -487,7 +493,9 @@ void InferenceRunner::TimeKernels(const float *deviceInputs, void *deviceResults
     if (binMs) *binMs = ms / runs;
   }
   WalkParams p = MakeWalkParams(walkInputs, rows);
-  p.out = finalize ? nullptr : static_cast<float *>(deviceResults);
+  p.s.fuseArgmax = fused ? 1 : 0;
+  p.out = finalize || (fused && ClassIdsAsInt8()) ? nullptr : static_cast<float *>(deviceResults);
+  p.classOut = fused && ClassIdsAsInt8() ? static_cast<int8_t *>(deviceResults) : nullptr;
   p.partial = finalize ? ws.partial : nullptr;
   Check(hipEventRecord(m_evStart, m_stream), "hipEventRecord");
   for (int i = 0; i < runs; ++i) Check(LaunchWalk(p, m_stream), "launch walk kernel");

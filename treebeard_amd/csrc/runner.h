@@ -109,6 +109,10 @@ private:
   // Rank-quantised plans: runs the binning kernel and returns the buffer the walk kernel reads.
   const float *PrepareRows(const float *deviceInputs, int64_t rows, uint8_t *ranks, hipStream_t stream);
   bool NeedsFinalize() const { return m_model.plan.treeSlices > 1 || m_forest.numClasses > 0; }
+  // Classifier, one tree slice, row-parallel LDS kernel: the walk kernel can store the class id itself.
+  bool FusesArgmax() const {
+    return m_forest.numClasses > 0 && m_model.plan.treeSlices == 1 && m_model.plan.kernel == LaunchPlan::Kernel::kRowParallelLds;
+  }
   WalkParams MakeWalkParams(const float *deviceInputs, int64_t rows) const;
   hipError_t LaunchWalk(const WalkParams &p, hipStream_t stream) const;
   void Launch(const float *deviceInputs, int64_t rows, float *out, int8_t *classOut, float *margins,
