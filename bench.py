@@ -96,7 +96,8 @@ def main():
     binding = "lds" if lds_time > hbm_time else "hbm"
     plan = runner.describe_plan()
     quantized = "quantizedRows=1" in plan
-    kernel = "WalkRowsLdsKernel" if "rows_lds" in plan else "WalkTreeParallelKernel"
+    kernel = ("WalkRowsTiledKernel" if " tileSize=1 " not in plan else "WalkRowsLdsKernel") if "rows_lds" in plan else \
+        ("WalkGlobalKernel" if "global_walk" in plan else "WalkTreeParallelKernel")
     # the rank-quantised path reads the f32 rows in its binning kernel: both kernels count for the HBM roofline
     hbm_ms = walk_ms + bin_ms if quantized else walk_ms
     hbm_gbs = hbm_bytes_row * rows / (hbm_ms * 1e-3) / 1e9
@@ -119,14 +120,8 @@ def main():
     # ... and the LDS: conflict-free reads of 4, 8 and 16 bytes per lane on every CU (the library's micro-benchmark)
     lds_measured = None
     if not args.copy_calibration:
-        import ctypes
-        from treebeard_amd.runtime_api import api
-        lds_measured = {}
-        for width in (4, 8, 16):
-            rate = ctypes.c_double()
-            if api().runtime_lib.tbmi_lds_read_bandwidth(width, ctypes.byref(rate)) != 0:
-                sys.exit("bench.py: " + api().last_error())
-            lds_measured["b%d" % (8 * width)] = rate.value / 1e9
+        from treebeard_amd.runtime_api import lds_read_bandwidth      # the bench-only library libtbamd_bench.so
+        lds_measured = {"b%d" % (8 * width): lds_read_bandwidth(width) / 1e9 for width in (4, 8, 16)}
     # What the LDS pipes need at those measured rates for this kernel's own mix (an 8-byte node read and a 4-byte
     # feature read per level, a 4-byte leaf read per tree): for the visited nodes only, and for the lock-step walk
     # that takes every row through the depth of each tree (the depth of the deepest tree of a bundle, in fact).
@@ -140,11 +135,32 @@ def main():
         lds_floor = {"visited_nodes_ms": visited_ms, "frac_of_visited_floor": visited_ms / walk_ms,
                      "lockstep_levels_per_row": depth_sum, "lockstep_ms": lockstep_ms,
                      "frac_of_lockstep_floor": lockstep_ms / walk_ms}
+    # HBM bytes per launch of the timed kernels, from rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this same command
+    # (scaled by a plain copy of known size); read from the committed summary, not measured in this run
     traffic = None
     traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(traffic_file):
         with open(traffic_file) as fh:
             traffic = json.load(fh).get("%s@%d" % (cfg.name, rows), {}).get("bytes_per_launch")
+
+    # The roofline that binds this workload (the larger of the two times above): LDS node + feature reads for the
+    # narrow models, HBM row streaming for the wide one.  `achieved` = algorithmic bytes per launch / the dominant
+    # kernel's launch duration (for the rank-quantised path the binning kernel reads the rows, so both count).
+    hbm_view = {"bound": "hbm", "achieved": hbm_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": hbm_gbs / HBM_PEAK_GBS,
+                "algorithmic_bytes_per_row": hbm_bytes_row, "measured_copy_gbs": copy_gbs,
+                "frac_of_measured_copy": hbm_gbs / copy_gbs if copy_gbs else None}
+    lds_view = {"bound": "lds", "achieved": lds_gbs, "peak": LDS_PEAK_GBS, "unit": "GB/s", "frac": lds_gbs / LDS_PEAK_GBS,
+                "algorithmic_bytes_per_row": lds_bytes_row, "visited_nodes_per_row": steps_per_row,
+                "measured_lds_read_gbs": lds_measured, "lds_floor": lds_floor,
+                "frac_of_measured_lds": (lds_gbs / lds_measured["b128"]) if lds_measured else None,
+                "peak_note": "256 CUs x 256 B/clk x 2.4 GHz; a scalar walk moves 10 B per lane per two LDS "
+                             "instructions of 2 clk each, so 62.5 % is its ceiling"}
+    roofline = dict(lds_view if binding == "lds" else hbm_view)
+    roofline.update({"traffic": traffic, "traffic_source": "profiles/hbm_traffic.json (rocprofv3 FETCH_SIZE + WRITE_SIZE "
+                                                           "of this command, scaled by a plain copy)" if traffic else None,
+                     "kernel": ("BinRowsKernel+" if quantized else "") + kernel,
+                     "kernel_ms": hbm_ms if binding == "hbm" else walk_ms,
+                     "walk_ms": walk_ms, "finalize_ms": fin_ms, "bin_ms": bin_ms, "path_ms": path_ms})
 
     line = {
         "metric": "rows/sec at 1 MI355X (2^20-row batch) + % of binding HBM/LDS roofline",
@@ -153,26 +169,8 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": cfg.name, "rows": rows, "trees": forest.num_trees, "features": cfg.num_features,
                    "objective": cfg.objective, "plan": plan},
-        "roofline": {"bound": "hbm", "achieved": hbm_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": hbm_gbs / HBM_PEAK_GBS, "traffic": traffic,
-                     "kernel": ("BinRowsKernel+" if quantized else "") + kernel,
-                     "kernel_ms": walk_ms, "finalize_ms": fin_ms, "bin_ms": bin_ms,
-                     "algorithmic_bytes_per_row": hbm_bytes_row,
-                     "binding": binding,       # which memory roofline binds this workload: see roofline_binding
-                     "measured_copy_gbs": copy_gbs,
-                     "frac_of_measured_copy": hbm_gbs / copy_gbs if copy_gbs else None},
-        "roofline_binding": {"bound": binding, "achieved": lds_gbs if binding == "lds" else hbm_gbs,
-                             "peak": LDS_PEAK_GBS if binding == "lds" else HBM_PEAK_GBS, "unit": "GB/s",
-                             "frac": (lds_gbs / LDS_PEAK_GBS) if binding == "lds" else (hbm_gbs / HBM_PEAK_GBS),
-                             "kernel": kernel, "kernel_ms": walk_ms, "path_ms": path_ms,
-                             "algorithmic_bytes_per_row": lds_bytes_row if binding == "lds" else hbm_bytes_row,
-                             "visited_nodes_per_row": steps_per_row,
-                             "measured_lds_read_gbs": lds_measured,
-                             "lds_floor": lds_floor,
-                             "frac_of_measured_lds": (lds_gbs / lds_measured["b128"]) if (lds_measured and binding == "lds") else None,
-                             "peak_note": "LDS: 256 CUs x 256 B/clk x 2.4 GHz (ds_read_b128 measured 237 B/clk/CU); "
-                                          "a scalar walk moves 10 B per lane per two LDS instructions (4 clk), so "
-                                          "62.5 % is its ceiling"},
+        "roofline": roofline,
+        "roofline_other": hbm_view if binding == "lds" else lds_view,   # the memory roofline that does not bind
     }
 
     if not args.no_cpu_baseline:

@@ -112,9 +112,6 @@ TBAMD_EXPORT void *findBestGPUScheduleAndCompileModel(void *tbContext);
 /* ------------------------------------------------------------------------ */
 TBAMD_EXPORT const char *tbmi_last_error(void);
 TBAMD_EXPORT int32_t tbmi_device_count(void);
-/* Micro-benchmark: bytes per second the device's LDS delivers for conflict-free reads of 4, 8 or 16 bytes per
- * lane (all CUs busy).  The walk kernels' LDS roofline is quoted against this measurement as well. */
-TBAMD_EXPORT int32_t tbmi_lds_read_bandwidth(int32_t widthBytes, double *bytesPerSecond);
 
 /* Inference on rows already resident in device memory (any row count); results as RunInference writes them.
  * The kernels run on a stream of the runner that does not order itself with any other stream: whatever

@@ -425,6 +425,4 @@ hipError_t LaunchFinalize(const FinalizeParams &p, hipStream_t) {
   return hipSuccess;
 }
 
-hipError_t MeasureLdsReadBandwidth(int, int, hipStream_t, double *) { return hipErrorNotSupported; }
-
 } // namespace tbamd

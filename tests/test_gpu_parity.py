@@ -753,14 +753,12 @@ def test_random_forests_and_plans(tmp_path, seed):
 
 
 def test_lds_micro_benchmark_reports_plausible_rates():
-    lib = api().runtime_lib
-    rates = {}
-    for width in (4, 8, 16):
-        rate = ctypes.c_double()
-        assert lib.tbmi_lds_read_bandwidth(width, ctypes.byref(rate)) == 0, api().last_error()
-        rates[width] = rate.value
+    """The bench-only library (libtbamd_bench.so, not part of the runtime library) that bench.py quotes."""
+    from treebeard_amd.runtime_api import lds_read_bandwidth
+    rates = {width: lds_read_bandwidth(width) for width in (4, 8, 16)}
     assert 1e13 < rates[4] < rates[8] <= 1.3 * rates[16] < 4e14          # tens to hundreds of TB/s on 256 CUs
-    assert lib.tbmi_lds_read_bandwidth(3, ctypes.byref(ctypes.c_double())) == -1
+    with pytest.raises(RuntimeError):
+        lds_read_bandwidth(3)
 
 
 @pytest.mark.parametrize("k,rows", [(2, 20000), (3, 9000), (1, 777)])
@@ -901,3 +899,35 @@ def test_profiled_runner_selects_the_same_leaves(synth_model, plain_file, tmp_pa
     runner = make_tiled_runner(higgs, hx.shape[0], tile_size, tiling_type, higgs_profile, peel)
     np.testing.assert_array_equal(gpu_leaf_ids(runner, hx), cpu_oracle.leaf_ids(hforest, hx))
     np.testing.assert_allclose(gpu_predict(runner, hx), data[:, -1], rtol=RTOL_SUM, atol=ATOL_PROB)
+
+
+@pytest.mark.parametrize("features,rows", [(20000, 300), (40000, 70)])
+def test_rows_too_wide_for_lds_walk_from_global_memory(tmp_path, features, rows):
+    """More features than a 16-bit byte offset inside an LDS row can address (the reference's default 16-bit
+    feature index allows 32767): the tuner falls back to the global-memory walk instead of refusing the model."""
+    rng = np.random.Generator(np.random.PCG64(features))
+    trees = [synth._grow_tree(rng, 6, lambda d, s: 0.85, lambda: (rng.integers(0, features), rng.normal()),
+                              lambda: rng.normal(0.0, 0.2)) for _ in range(40)]
+    path = tmp_path / "wide.json"
+    synth.write_xgboost_json(path, trees, features)
+    forest = model_io.load_xgboost_json(path)
+    x = rng.normal(size=(rows, features)).astype(np.float32)
+    runner = make_runner(path, rows)
+    assert "kernel=global_walk" in runner.describe_plan()
+    check_against_oracle(runner, forest, x)
+
+
+def test_time_kernels_leaves_the_outputs_of_one_run(synth_model):
+    """Repeated launches inside tbmi_time_kernels (wide finalize of a sliced classifier included) leave the same
+    results as one tbmi_run_device."""
+    rows = 50
+    x = synth.CONFIGS[3].batch_rows(rows, seed_offset=2)
+    runner = make_runner(synth_model(3), rows)
+    runner.set_plan(64, 2, 2, 8192, 24)
+    assert "treeSlices=24" in runner.describe_plan()
+    expected = gpu_predict(runner, x)
+    dx = torch.from_numpy(x).cuda()
+    out = torch.full((rows,), -1, dtype=torch.int8, device="cuda")
+    torch.cuda.synchronize()
+    runner.time_kernels(dx.data_ptr(), out.data_ptr(), rows, 3)
+    np.testing.assert_array_equal(out.cpu().numpy(), expected)

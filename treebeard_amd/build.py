@@ -1,4 +1,5 @@
-"""Builds the runtime library (libtreebeard_amd.so) in-tree with hipcc for gfx950."""
+"""Builds the runtime library (libtreebeard_amd.so) and the bench-only micro-benchmark library
+(libtbamd_bench.so) in-tree with hipcc for gfx950."""
 import os
 import subprocess
 import sys
@@ -6,6 +7,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtreebeard_amd.so")
+BENCH_LIB = os.path.join(HERE, "libtbamd_bench.so")
 SOURCES = ["forest.cpp", "json_reader.cpp", "xgboost_loader.cpp", "onnx_loader.cpp", "packer.cpp", "tuner.cpp", "model_file.cpp",
            "host_copy.cpp", "runner.cpp", "runtime.cpp", "kernels.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -36,6 +38,11 @@ def build(verbose=False):
     if failed:
         raise RuntimeError("hipcc failed")
     subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs, check=True)
+    bench = subprocess.run([HIPCC] + FLAGS + ["-shared", os.path.join(CSRC, "bench_kernels.hip"), "-o", BENCH_LIB],
+                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if bench.returncode != 0:
+        sys.stderr.write("== bench_kernels.hip failed ==\n%s\n" % bench.stdout)
+        raise RuntimeError("hipcc failed")
     return LIB
 
 

@@ -44,8 +44,12 @@ struct WalkParams {
   const int32_t *slotTree = nullptr;
 };
 
+// From this many tree slices on, small batches are finalized by a wave per (row, class); classifiers then need
+// one spare slot of [rows][classes] doubles behind the last slice of the partial sums.
+constexpr int kWideFinalizeSlices = 16;
+
 struct FinalizeParams {
-  double *partial = nullptr;   // [slices][rows][max(1, classes)]; the wide finalize parks class sums in slice 0
+  double *partial = nullptr;   // [slices (+ 1 spare, see kWideFinalizeSlices)][rows][max(1, classes)]
   int64_t rows = 0;
   int32_t numClasses = 0;
   int32_t treeSlices = 1;      // number of partial sums per (row, class)
@@ -75,7 +79,5 @@ hipError_t LaunchWalkTreeParallel(const WalkParams &p, int interleave, size_t ld
 // one per row; p.globalNodes / p.globalTrees instead of groups and bundles.
 hipError_t LaunchWalkGlobal(const WalkParams &p, int interleave, hipStream_t stream);
 hipError_t LaunchFinalize(const FinalizeParams &p, hipStream_t stream);
-// Conflict-free LDS reads of 4, 8 or 16 bytes per lane on every CU: the measured bytes per second.
-hipError_t MeasureLdsReadBandwidth(int widthBytes, int computeUnits, hipStream_t stream, double *bytesPerSecond);
 
 } // namespace tbamd

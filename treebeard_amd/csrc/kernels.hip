@@ -963,7 +963,7 @@ __global__ void __launch_bounds__(256) FinalizeKernel(const FinalizeParams p) {
   }
 }
 
-// Small batches split over many tree slices: one wave per (row, class).  The lanes fetch the slice
+// Small batches split over many tree slices (kWideFinalizeSlices or more): one wave per (row, class).  The lanes fetch the slice
 // partials side by side (one memory latency instead of one per slice), each adds its slices in slice
 // order, and a fixed butterfly combines the lanes - the order of additions depends only on the number
 // of slices.
@@ -982,8 +982,9 @@ __global__ void __launch_bounds__(256) FinalizeWideKernel(const FinalizeParams p
     if (lane == 0) p.out[row] = (float)(p.transform == 1 ? 1.0 / (1.0 + exp(-margin)) : margin);
     return;
   }
-  // classifiers: park the class sum in the first slice's slot; FinalizeKernel (1 slice) does the rest
-  if (lane == 0) p.partial[row * Cn + c] = margin - p.initialValue;
+  // classifiers: the class sum goes into the spare slot behind the last slice; FinalizeKernel (1 slice, reading
+  // that slot) does the rest.  The slices themselves stay as they are, so the launch can be repeated.
+  if (lane == 0) p.partial[((int64_t)p.treeSlices * p.rows + row) * Cn + c] = margin - p.initialValue;
 }
 
 // The ceiling on dynamic LDS is an attribute of each kernel: it is raised once per kernel, to the whole
@@ -1228,86 +1229,17 @@ hipError_t LaunchBinRows(const float *x, const float *table, uint8_t *ranks, int
 #undef TBAMD_BIN_CASE
 }
 
-// ---------------------------------------------------------------------------
-// LDS read micro-benchmark: what the LDS pipes of this device deliver for conflict-free reads of 4, 8
-// and 16 bytes per lane (lane i reads bank-aligned element i of a row; eight independent rows per
-// iteration).  The walk kernels are priced against these figures rather than a datasheet's.
-// ---------------------------------------------------------------------------
-namespace {
-template <int kWidth>
-__global__ void __launch_bounds__(1024) LdsReadBenchKernel(int iterations, uint32_t *sink) {
-  extern __shared__ __align__(16) unsigned char lds[];
-  for (int i = threadIdx.x; i < 16384; i += blockDim.x) reinterpret_cast<uint32_t *>(lds)[i] = (uint32_t)i;
-  __syncthreads();
-  const uint32_t lane = threadIdx.x & 63u;
-  uint32_t address[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) address[i] = (lane * kWidth + (uint32_t)i * 64u * kWidth) & 0xFFFFu;
-  uint32_t issued = 0;
-  for (int it = 0; it < iterations; ++it) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      if (kWidth == 4) {
-        uint32_t v;
-        asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(7)" : "=v"(v) : "v"(address[i]));
-      } else if (kWidth == 8) {
-        uint64_t v;
-        asm volatile("ds_read_b64 %0, %1\n\ts_waitcnt lgkmcnt(7)" : "=v"(v) : "v"(address[i]));
-      } else {
-        __uint128_t v;
-        asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(7)" : "=v"(v) : "v"(address[i]));
-      }
-      ++issued;
-    }
-  }
-  asm volatile("s_waitcnt lgkmcnt(0)");
-  if (issued == 0x7FFFFFFFu) sink[0] = issued; // (never true: keeps the loop alive)
-}
-} // namespace
-
-hipError_t MeasureLdsReadBandwidth(int widthBytes, int computeUnits, hipStream_t stream, double *bytesPerSecond) {
-  if (!bytesPerSecond || computeUnits < 1 || (widthBytes != 4 && widthBytes != 8 && widthBytes != 16)) return hipErrorInvalidValue;
-  const int blocks = computeUnits * 2, threads = 1024, iterations = 2000;
-  uint32_t *sink = nullptr;
-  hipError_t e = hipMalloc(reinterpret_cast<void **>(&sink), sizeof(uint32_t));
-  if (e != hipSuccess) return e;
-  hipEvent_t start = nullptr, stop = nullptr;
-  auto launch = [&](int it) {
-    if (widthBytes == 4) LdsReadBenchKernel<4><<<blocks, threads, 65536, stream>>>(it, sink);
-    else if (widthBytes == 8) LdsReadBenchKernel<8><<<blocks, threads, 65536, stream>>>(it, sink);
-    else LdsReadBenchKernel<16><<<blocks, threads, 65536, stream>>>(it, sink);
-  };
-  float ms = 0.f;
-  e = hipEventCreate(&start);
-  if (e == hipSuccess) e = hipEventCreate(&stop);
-  if (e == hipSuccess) {
-    launch(10); // warm-up
-    e = hipEventRecord(start, stream);
-    launch(iterations);
-    if (e == hipSuccess) e = hipEventRecord(stop, stream);
-    if (e == hipSuccess) e = hipEventSynchronize(stop);
-    if (e == hipSuccess) e = hipEventElapsedTime(&ms, start, stop);
-    if (e == hipSuccess) e = hipGetLastError();
-  }
-  if (start) (void)hipEventDestroy(start);
-  if (stop) (void)hipEventDestroy(stop);
-  (void)hipFree(sink);
-  if (e != hipSuccess) return e;
-  const double bytes = (double)blocks * threads * iterations * 8.0 * widthBytes;
-  *bytesPerSecond = bytes / (ms * 1e-3);
-  return hipSuccess;
-}
-
 hipError_t LaunchFinalize(const FinalizeParams &p, hipStream_t stream) {
   if (p.rows <= 0) return hipSuccess;
   const int Cn = p.numClasses > 0 ? p.numClasses : 1;
   FinalizeParams q = p;
-  if (p.treeSlices >= 16 && p.rows * Cn <= 65536) { // few rows, many slices: a wave per (row, class)
+  if (p.treeSlices >= kWideFinalizeSlices && p.rows * Cn <= 65536) { // few rows, many slices: a wave per (row, class)
     const int64_t waves = p.rows * Cn;
     FinalizeWideKernel<<<dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream>>>(p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || p.numClasses == 0) return e;
-    q.treeSlices = 1; // the class sums now sit in slice 0
+    q.partial = p.partial + (int64_t)p.treeSlices * p.rows * Cn; // the class sums now sit in the spare slot
+    q.treeSlices = 1;
   }
   const int64_t blocks = (q.rows + 255) / 256;
   FinalizeKernel<<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(q);

@@ -179,7 +179,10 @@ void InferenceRunner::Repack(const LaunchPlan &plan) {
 
 size_t InferenceRunner::PartialBytes(int64_t rows) const {
   if (!NeedsFinalize()) return 0;
-  return (size_t)m_model.PartialCount() * (size_t)rows * (size_t)std::max(1, m_forest.numClasses) * sizeof(double);
+  // (+ the spare slot the wide finalize of a classifier leaves its class sums in)
+  const size_t slots = (size_t)m_model.PartialCount() +
+                       (m_forest.numClasses > 0 && m_model.PartialCount() >= kWideFinalizeSlices ? 1 : 0);
+  return slots * (size_t)rows * (size_t)std::max(1, m_forest.numClasses) * sizeof(double);
 }
 
 size_t InferenceRunner::RanksBytes(int64_t rows) const {

@@ -345,20 +345,6 @@ int32_t tbmi_run_host(intptr_t h, const void *in, void *out, int64_t rows) {
       -1);
 }
 
-int32_t tbmi_lds_read_bandwidth(int32_t widthBytes, double *bytesPerSecond) {
-  return Guard(
-      [&] {
-        int devices = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDeviceCount(&devices) != hipSuccess || devices == 0) throw Error("no HIP device available");
-        if (hipGetDeviceProperties(&prop, 0) != hipSuccess) throw Error("hipGetDeviceProperties failed");
-        const hipError_t e = MeasureLdsReadBandwidth(widthBytes, prop.multiProcessorCount, nullptr, bytesPerSecond);
-        if (e != hipSuccess) throw Error(std::string("LDS micro-benchmark: ") + hipGetErrorString(e));
-        return 0;
-      },
-      -1);
-}
-
 int32_t tbmi_result_bytes(intptr_t h) { return Guard([&] { return Runner(h)->ReturnTypeBytes(); }, -1); }
 
 int32_t tbmi_run_device_multiclass(intptr_t h, const float *in, int64_t rows, int8_t *cls, float *margins,

@@ -134,8 +134,9 @@ LaunchPlan ChooseScalarPlan(const Forest &forest, int64_t batchSize, const GPUAu
     plan.treeSlices = (int32_t)std::max<int64_t>(1, slices);
     return plan;
   }
-  if ((BiggestTreeNodes(forest) + 2) * kNodeBytes > 65536) {
-    // A tree that cannot sit in one LDS group: walk from global memory.
+  // A tree that cannot sit in one LDS group walks from global memory; so do rows that neither LDS form can
+  // hold (below): more than 16383 features have no 16-bit byte offset inside one row-major LDS row.
+  auto globalPlan = [&]() {
     LaunchPlan plan;
     plan.kernel = LaunchPlan::Kernel::kGlobalWalk;
     plan.rowsPerBlock = 256;
@@ -148,13 +149,17 @@ LaunchPlan ChooseScalarPlan(const Forest &forest, int64_t batchSize, const GPUAu
     plan.treeSlices = (int32_t)std::max<int64_t>(1, std::min<int64_t>(slices, (int64_t)forest.trees.size()));
     plan.groupBytes = 0;
     return plan;
-  }
+  };
+  if ((BiggestTreeNodes(forest) + 2) * kNodeBytes > 65536) return globalPlan();
+  const bool rowMajorFits = (int64_t)(forest.numFeatures + 1) * 4 <= 0xFFFF &&
+                            (int64_t)(forest.numFeatures + 1) * 4 + (BiggestTreeNodes(forest) + 2) * kNodeBytes + 4096 <=
+                                limits.ldsBytesPerBlock;
   bool fitsTransposed = false;
   {
     bool words = false;
     fitsTransposed = RowTileFits(forest.numFeatures, 64, limits.ldsBytesPerBlock, &words);
   }
-  if (batchSize > 0 && batchSize <= 128) return ChooseTreeParallelPlan(forest, batchSize, ov, limits);
+  if (batchSize > 0 && batchSize <= 128 && rowMajorFits) return ChooseTreeParallelPlan(forest, batchSize, ov, limits);
   if (!fitsTransposed) {
     // Rows too wide for 64 f32 rows in LDS: one-byte ranks (exact) if every feature has few enough
     // distinct thresholds and 64 rank rows fit; otherwise a few f32 rows with several lanes each.
@@ -181,7 +186,7 @@ LaunchPlan ChooseScalarPlan(const Forest &forest, int64_t batchSize, const GPUAu
       plan.treeSlices = (int32_t)std::max<int64_t>(1, slices);
       return plan;
     }
-    return ChooseTreeParallelPlan(forest, batchSize, ov, limits);
+    return rowMajorFits ? ChooseTreeParallelPlan(forest, batchSize, ov, limits) : globalPlan();
   }
 
   LaunchPlan plan;

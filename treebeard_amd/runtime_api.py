@@ -61,7 +61,6 @@ SIGNATURES = {
     "tbmi_time_kernels": (c_i32, [c_ip, c_vp, c_vp, c_i64, c_i32, ctypes.POINTER(ctypes.c_double),
                                   ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]),
     "tbmi_result_bytes": (c_i32, [c_ip]),
-    "tbmi_lds_read_bandwidth": (c_i32, [c_i32, ctypes.POINTER(ctypes.c_double)]),
     "tbmi_run_host": (c_i32, [c_ip, c_vp, c_vp, c_i64]),
     "tbmi_set_global_walk_plan": (c_i32, [c_ip, c_i32, c_i32, c_i32]),
     "tbmi_set_quantized_plan": (c_i32, [c_ip, c_i32, c_i32, c_i32, c_i32]),
@@ -99,6 +98,24 @@ class TreebeardAPI:
     def last_error(self):
         msg = self.runtime_lib.tbmi_last_error()
         return msg.decode() if msg else ""
+
+
+BENCH_LIB_PATH = os.path.join(_HERE, "libtbamd_bench.so")
+
+
+def lds_read_bandwidth(width_bytes):
+    """Bytes per second of conflict-free LDS reads (4, 8 or 16 bytes per lane) measured by the bench-only
+    library libtbamd_bench.so; raises when that library is missing or the measurement fails."""
+    if not os.path.exists(BENCH_LIB_PATH):
+        raise FileNotFoundError("%s is missing: build it with `python -m treebeard_amd.build`" % BENCH_LIB_PATH)
+    lib = ctypes.CDLL(BENCH_LIB_PATH)
+    lib.tbbench_lds_read_bandwidth.restype = c_i32
+    lib.tbbench_lds_read_bandwidth.argtypes = [c_i32, ctypes.POINTER(ctypes.c_double)]
+    rate = ctypes.c_double()
+    rc = lib.tbbench_lds_read_bandwidth(width_bytes, ctypes.byref(rate))
+    if rc != 0:
+        raise RuntimeError("LDS micro-benchmark failed with HIP error %d" % rc)
+    return rate.value
 
 
 _api = None
