@@ -580,7 +580,26 @@ WalkRowsTiledKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes
 // 64 of them into LDS, and when the batch has too few rows to fill the chip
 // with one lane per row.
 // ---------------------------------------------------------------------------
+// One butterfly step on doubles.  Partners 1, 2, 4 and 8 lanes away are reached with DPP operand swizzles
+// inside the VALU (quad permutes, the mirror of half a row and of a row: after the steps before them every
+// lane of the mirrored group already holds the same partial sum, so the mirror partner is as good as the
+// xor partner); only the steps across rows of 16 lanes go through the LDS crossbar (ds_bpermute).
+template <int kDppCtrl>
+__device__ __forceinline__ double DppMove(double v) {
+  int lo = __double2loint(v), hi = __double2hiint(v);
+  lo = __builtin_amdgcn_update_dpp(0, lo, kDppCtrl, 0xF, 0xF, false);
+  hi = __builtin_amdgcn_update_dpp(0, hi, kDppCtrl, 0xF, 0xF, false);
+  return __hiloint2double(hi, lo);
+}
+
 __device__ __forceinline__ double ShuffleXor(double v, int mask) {
+  switch (mask) {
+  case 1: return DppMove<0xB1>(v);  // quad_perm [1,0,3,2]
+  case 2: return DppMove<0x4E>(v);  // quad_perm [2,3,0,1]
+  case 4: return DppMove<0x141>(v); // row_half_mirror
+  case 8: return DppMove<0x140>(v); // row_mirror
+  default: break;
+  }
   int lo = __double2loint(v), hi = __double2hiint(v);
   lo = __shfl_xor(lo, mask, 64);
   hi = __shfl_xor(hi, mask, 64);
@@ -691,7 +710,7 @@ WalkTreeParallelKernel(const float *__restrict__ x, const uint4 *__restrict__ no
 
       // combine the lanes of each row: butterfly inside the wave ...
       const int inWave = TL < 64 ? TL : 64;
-      for (int m = inWave >> 1; m >= 1; m >>= 1) acc += ShuffleXor(acc, m);
+      for (int m = 1; m < inWave; m <<= 1) acc += ShuffleXor(acc, m); // (ascending: see ShuffleXor)
       if (TL > 64) { // ... then across the row's waves through LDS
         __syncthreads();
         if ((tid & 63) == 0) waveScratch[tid >> 6] = acc;
@@ -976,7 +995,7 @@ __global__ void __launch_bounds__(256) FinalizeWideKernel(const FinalizeParams p
   const int c = (int)(item - row * Cn);
   double sum = 0.0;
   for (int s = lane; s < p.treeSlices; s += 64) sum += p.partial[((int64_t)s * p.rows + row) * Cn + c];
-  for (int m = 32; m >= 1; m >>= 1) sum += ShuffleXor(sum, m);
+  for (int m = 1; m <= 32; m <<= 1) sum += ShuffleXor(sum, m); // (ascending: see ShuffleXor)
   const double margin = p.initialValue + sum;
   if (p.numClasses == 0) {
     if (lane == 0) p.out[row] = (float)(p.transform == 1 ? 1.0 / (1.0 + exp(-margin)) : margin);
