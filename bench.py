@@ -30,6 +30,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (default: the headline, 2)")
     ap.add_argument("--rows", type=int, default=0, help="override the batch size")
+    ap.add_argument("--tile-size", type=int, default=1, help="CompilerOptions tile size (2, 3, 4 run the tiled walk kernel)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--autotune", action="store_true", help="timed launch-plan search before measuring")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU-baseline duration")
@@ -49,7 +50,7 @@ def main():
     cache = os.path.join(tempfile.gettempdir(), "treebeard_amd_models")
     model = synth.model_path(args.config, cache)
     x = cfg.batch_rows(rows)
-    options = treebeard.CompilerOptions(rows, 1)
+    options = treebeard.CompilerOptions(rows, args.tile_size)
     if cfg.num_class > 0:                       # class ids as int8, the reference's multiclass setting
         options.SetReturnTypeWidth(8)
         options.SetReturnTypeIsFloatType(False)

@@ -35,6 +35,7 @@ struct WalkParams {
   const DeviceGroup *groups = nullptr;
   const DeviceGlobalNode *globalNodes = nullptr; // global-memory walk only
   const DeviceGlobalTree *globalTrees = nullptr;
+  bool peelWalks = false;         // bundles carry peel depths below their depths: use the kernels that look at them
   float *out = nullptr;           // used when the epilogue is fused (1 slice; class ids as float32 with fuseArgmax)
   int8_t *classOut = nullptr;     // fuseArgmax: class ids as int8 (out is then null)
   double *partial = nullptr;      // [partials][rows][max(1, classes)] otherwise

@@ -114,7 +114,17 @@ __device__ __forceinline__ void StageRows(const float *__restrict__ src, int val
 // without growing the row tile; their sums meet in an LDS cross-wave pass.
 // Sums are kept in double; trees are added in packed order.
 // ---------------------------------------------------------------------------
-template <int K, int PF, int kMode, bool kDump>
+// kPeel: bundles carry a peel depth taken from a hit-count profile (the steps that bring 90 % of the profiled
+// rows to a leaf, src/mlir/ProbabilityBasedTilingTransform.cpp:66-73): the walk takes that many steps blind and
+// then goes on only while some lane of the wave still moves, at most to the full depth.  Without kPeel the
+// peel depth is not looked at and every bundle walks its full depth.
+//
+// kVariant picks what is compiled in beside the plain walk (each costs the plain walk about a percent when it
+// is merely present): kWalkDump the leaf-id dump of the parity checks, kWalkPeel the peeled walk, kWalkFuse the
+// classifiers' running arg-max (WalkScalars::fuseArgmax).
+enum WalkVariant : int { kWalkPlain = 0, kWalkDump = 1, kWalkPeel = 2, kWalkFuse = 3 };
+
+template <int K, int PF, int kMode, int kVariant>
 __global__ void __launch_bounds__(1024)
 WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16,
                   const DeviceBundle *__restrict__ bundles, const DeviceNode *__restrict__ bundleRoots,
@@ -122,6 +132,7 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
                   const WalkScalars s, float *__restrict__ out, int8_t *__restrict__ classOut,
                   double *__restrict__ partial, int32_t *__restrict__ leafIds, const int32_t *__restrict__ nodeOrigin,
                   const int32_t *__restrict__ slotTree) {
+  constexpr bool kDump = kVariant == kWalkDump, kPeel = kVariant == kWalkPeel, kFuse = kVariant == kWalkFuse;
   // LDS: [tree group nodes | transposed row tile].  The group sits at LDS
   // address 0 so that node pointers are LDS addresses as stored.
   extern __shared__ __align__(16) unsigned char lds[];
@@ -210,7 +221,7 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
         for (int t = 0; t < TT; ++t) acc += meet[t * RB + lane];                                                       \
       }                                                                                                                \
     }                                                                                                                  \
-    if (s.fuseArgmax) {                                                                                                \
+    if (kFuse) {                                                                                                       \
       /* running arg-max with the generated code's tie rule (replace unless strictly greater); a class */              \
       /* without trees scores the initial value */                                                                     \
       const float m = (float)(s.initialValue + acc);                                                                   \
@@ -276,8 +287,7 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
             addr[k] = (root.meta >> 16) + (left ? 0u : kNodeBytes);
           }
         }
-        // bd.peelDepth (== depth unless a hit-count profile asked for peeled walks) steps are taken blind ...
-        const int blind = (int)bd.peelDepth;
+        const int blind = kPeel ? (int)bd.peelDepth : depth;
 #pragma unroll 2
         for (int d = kMode != kTileRankU8 ? 1 : 0; d < blind; ++d) {
 #pragma unroll
@@ -290,21 +300,22 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
             addr[k] = (node.y >> 16) + (left ? 0u : kNodeBytes);
           }
         }
-        // ... and the rest only while some lane of the wave still moves (leaves point at themselves)
-        for (int d = blind > 1 || kMode == kTileRankU8 ? blind : 1; d < depth; ++d) {
-          bool moved = false;
+        if (kPeel) { // the rest only while some lane of the wave still moves (leaves point at themselves)
+          for (int d = blind > 1 || kMode == kTileRankU8 ? blind : 1; d < depth; ++d) {
+            bool moved = false;
 #pragma unroll
-          for (int k = 0; k < K; ++k) {
-            const U32x2 node = LdsLoadNode(addr[k]);
-            const uint32_t off = kMode == kTileF32Bytes ? (node.y & 0xFFFFu) : (node.y & 0xFFFFu) << 2;
-            bool left;
-            if (kMode == kTileRankU8) left = LdsLoadByte(column + off) <= node.x;
-            else left = LdsLoadFloat(column + off) < AsFloat(node.x);
-            const uint32_t next = (node.y >> 16) + (left ? 0u : kNodeBytes);
-            moved = moved || next != addr[k];
-            addr[k] = next;
+            for (int k = 0; k < K; ++k) {
+              const U32x2 node = LdsLoadNode(addr[k]);
+              const uint32_t off = kMode == kTileF32Bytes ? (node.y & 0xFFFFu) : (node.y & 0xFFFFu) << 2;
+              bool left;
+              if (kMode == kTileRankU8) left = LdsLoadByte(column + off) <= node.x;
+              else left = LdsLoadFloat(column + off) < AsFloat(node.x);
+              const uint32_t next = (node.y >> 16) + (left ? 0u : kNodeBytes);
+              moved = moved || next != addr[k];
+              addr[k] = next;
+            }
+            if (!__any(moved)) break;
           }
-          if (!__any(moved)) break;
         }
 #pragma unroll
         for (int k = 0; k < K; ++k) acc += (double)LdsLoadFloat(addr[k]);
@@ -324,7 +335,7 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
 
   if (C > 0) {
     TBAMD_FLUSH_CLASS(C)
-    if (s.fuseArgmax && tt == 0 && lane < valid) {
+    if (kFuse && tt == 0 && lane < valid) {
       if (classOut) classOut[row] = (int8_t)bestClass;
       else out[row] = (float)bestClass;
     }
@@ -1014,20 +1025,25 @@ template <auto Kernel> hipError_t AllowFullLds() {
   return status;
 }
 
+template <int K, int PF, int W, int V>
+hipError_t LaunchWalkVariant(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
+  hipError_t e = AllowFullLds<&WalkRowsLdsKernel<K, PF, W, V>>();
+  if (e != hipSuccess) return e;
+  WalkRowsLdsKernel<K, PF, W, V><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.bundleRoots, p.groups, p.s, p.out, p.classOut,
+                                                                    p.partial, p.leafIds, p.nodeOrigin, p.slotTree);
+  return hipGetLastError();
+}
+
 template <int K, int PF, int W>
 hipError_t LaunchWalkKP(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
-  if (p.leafIds) {
-    hipError_t e = AllowFullLds<&WalkRowsLdsKernel<K, PF, W, true>>();
-    if (e != hipSuccess) return e;
-    WalkRowsLdsKernel<K, PF, W, true><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.bundleRoots, p.groups, p.s, p.out,
-                                                                         p.classOut, p.partial, p.leafIds, p.nodeOrigin, p.slotTree);
-  } else {
-    hipError_t e = AllowFullLds<&WalkRowsLdsKernel<K, PF, W, false>>();
-    if (e != hipSuccess) return e;
-    WalkRowsLdsKernel<K, PF, W, false><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.bundleRoots, p.groups, p.s, p.out,
-                                                                          p.classOut, p.partial, nullptr, nullptr, nullptr);
+  if (p.leafIds) { // (the dump kernel walks every bundle to its full depth and leaves the arg-max to the finalize kernel)
+    if (p.s.fuseArgmax) return hipErrorInvalidValue;
+    return LaunchWalkVariant<K, PF, W, kWalkDump>(p, grid, block, ldsBytes, stream);
   }
-  return hipGetLastError();
+  if (p.s.fuseArgmax) return LaunchWalkVariant<K, PF, W, kWalkFuse>(p, grid, block, ldsBytes, stream);
+  // peeled walks are built for the f32 tile with byte offsets only; elsewhere every bundle walks its full depth
+  if (p.peelWalks && W == kTileF32Bytes) return LaunchWalkVariant<K, PF, kTileF32Bytes, kWalkPeel>(p, grid, block, ldsBytes, stream);
+  return LaunchWalkVariant<K, PF, W, kWalkPlain>(p, grid, block, ldsBytes, stream);
 }
 
 template <int K, int W>

@@ -266,6 +266,7 @@ WalkParams InferenceRunner::MakeWalkParams(const float *deviceInputs, int64_t ro
   p.s.rowsPerBlock = m_model.plan.rowsPerBlock;
   p.s.treeLanes = m_model.plan.treeLanes;
   p.s.initialValue = m_forest.initialValue;
+  p.peelWalks = m_model.plan.peelWalks;
   p.x = deviceInputs;
   p.globalNodes = m_dGlobalNodes;
   p.globalTrees = m_dGlobalTrees;
@@ -282,7 +283,7 @@ void InferenceRunner::Launch(const float *deviceInputs, int64_t rows, float *out
   WalkParams p = MakeWalkParams(PrepareRows(deviceInputs, rows, ws.ranks, stream), rows);
   // A classifier whose trees all sit in one slice needs no second kernel when only the class id is wanted:
   // the row-parallel kernels keep the running arg-max themselves.
-  const bool fused = FusesArgmax() && !margins && !probabilities;
+  const bool fused = FusesArgmax() && !margins && !probabilities && !leafIds;
   const bool finalize = NeedsFinalize() && !fused;
   p.s.fuseArgmax = fused ? 1 : 0;
   p.out = finalize ? nullptr : out;
