@@ -413,13 +413,14 @@ __device__ __forceinline__ uint32_t TileStep(uint32_t addr, uint32_t column) {
   return childBase + child * TileBytes(T);
 }
 
-template <int T, int K, int PF, bool kDump>
+template <int T, int K, int PF, int kVariant> // kVariant: kWalkPlain, kWalkDump or kWalkFuse (the peel tail is always there)
 __global__ void __launch_bounds__(1024)
 WalkRowsTiledKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16,
                     const DeviceBundle *__restrict__ bundles, const DeviceGroup *__restrict__ groups,
                     const WalkScalars s, float *__restrict__ out, int8_t *__restrict__ classOut,
                     double *__restrict__ partial, int32_t *__restrict__ leafIds, const int32_t *__restrict__ nodeOrigin,
                     const int32_t *__restrict__ slotTree) {
+  constexpr bool kDump = kVariant == kWalkDump, kFuse = kVariant == kWalkFuse;
   extern __shared__ __align__(16) unsigned char lds[];
   const int tid = threadIdx.x;
   const int threads = blockDim.x;
@@ -471,7 +472,7 @@ WalkRowsTiledKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes
         for (int t = 0; t < TT; ++t) acc += meet[t * RB + lane];                                                       \
       }                                                                                                                \
     }                                                                                                                  \
-    if (s.fuseArgmax) {                                                                                                \
+    if (kFuse) {                                                                                                \
       /* running arg-max with the generated code's tie rule (replace unless strictly greater); a class */              \
       /* without trees scores the initial value */                                                                     \
       const float m = (float)(s.initialValue + acc);                                                                   \
@@ -555,7 +556,7 @@ WalkRowsTiledKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes
 
   if (C > 0) {
     TBAMD_FLUSH_CLASS(C)
-    if (s.fuseArgmax && tt == 0 && lane < valid) {
+    if (kFuse && tt == 0 && lane < valid) {
       if (classOut) classOut[row] = (int8_t)bestClass;
       else out[row] = (float)bestClass;
     }
@@ -1099,20 +1100,23 @@ hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, int tileMode, 
 }
 
 namespace {
+template <int T, int K, int PF, int V>
+hipError_t LaunchTiledVariant(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
+  hipError_t e = AllowFullLds<&WalkRowsTiledKernel<T, K, PF, V>>();
+  if (e != hipSuccess) return e;
+  WalkRowsTiledKernel<T, K, PF, V><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out, p.classOut, p.partial,
+                                                                      p.leafIds, p.nodeOrigin, p.slotTree);
+  return hipGetLastError();
+}
+
 template <int T, int K, int PF>
 hipError_t LaunchTiledTKP(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
   if (p.leafIds) {
-    hipError_t e = AllowFullLds<&WalkRowsTiledKernel<T, K, PF, true>>();
-    if (e != hipSuccess) return e;
-    WalkRowsTiledKernel<T, K, PF, true><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out, p.classOut,
-                                                                          p.partial, p.leafIds, p.nodeOrigin, p.slotTree);
-  } else {
-    hipError_t e = AllowFullLds<&WalkRowsTiledKernel<T, K, PF, false>>();
-    if (e != hipSuccess) return e;
-    WalkRowsTiledKernel<T, K, PF, false><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out, p.classOut,
-                                                                           p.partial, nullptr, nullptr, nullptr);
+    if (p.s.fuseArgmax) return hipErrorInvalidValue;
+    return LaunchTiledVariant<T, K, PF, kWalkDump>(p, grid, block, ldsBytes, stream);
   }
-  return hipGetLastError();
+  if (p.s.fuseArgmax) return LaunchTiledVariant<T, K, PF, kWalkFuse>(p, grid, block, ldsBytes, stream);
+  return LaunchTiledVariant<T, K, PF, kWalkPlain>(p, grid, block, ldsBytes, stream);
 }
 
 template <int T, int K>
