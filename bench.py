@@ -23,6 +23,27 @@ HBM_PEAK_GBS = 8000.0                      # MI355X HBM3E, published
 LDS_PEAK_GBS = 256 * 256 * 2.4             # 256 CUs x 256 B/clk x 2.4 GHz = 157 286 GB/s, nominal
 
 
+def print_lds_read_costs():
+    """Table of cycles per wave-level LDS read per compute unit (nominal shader clock), from the bench-only library."""
+    import torch                                                  # initialises the device the library measures on
+    from treebeard_amd.runtime_api import LDS_READ_OPS, lds_read_cost
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU")
+    patterns = [(0, "lane i reads element i"), (1, "random over 48 KB"), (2, "random over 1 KB"),
+                (5, "random among 32 elements"), (6, "random among 64 elements"), (7, "random among 128 elements")]
+    masks = ["all lanes", "lanes 0-31", "even lanes", "random half", "random quarter"]
+    print("| instruction | address pattern | lanes active | cycles per read per CU |")
+    print("|---|---|---|---|")
+    for op, name in enumerate(LDS_READ_OPS):
+        for pattern, pattern_name in patterns:
+            if pattern >= 5 and name not in ("ds_read_b32", "ds_read_b64", "ds_read2_b32"):
+                continue
+            for mask, mask_name in enumerate(masks):
+                if mask > 0 and name not in ("ds_read_b32", "ds_read_b64"):
+                    continue
+                print("| %s | %s | %s | %.2f |" % (name, pattern_name, mask_name, lds_read_cost(op, pattern, mask)), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -36,7 +57,11 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU-baseline duration")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="also run one plain device copy of this many MiB (counter calibration for rocprofv3 --pmc)")
+    ap.add_argument("--lds-read-costs", action="store_true",
+                    help="print what the LDS of this device charges per wave-level read (instruction x address pattern x exec mask) and exit")
     args = ap.parse_args()
+    if args.lds_read_costs:
+        return print_lds_read_costs()
     if args.gpus != 1:
         sys.exit("bench.py: this engine runs on ONE GPU (a batch would shard by rows, each GPU holding the whole model) - use --gpus 1")
 

@@ -759,6 +759,13 @@ def test_lds_micro_benchmark_reports_plausible_rates():
     assert 1e13 < rates[4] < rates[8] <= 1.3 * rates[16] < 4e14          # tens to hundreds of TB/s on 256 CUs
     with pytest.raises(RuntimeError):
         lds_read_bandwidth(3)
+    from treebeard_amd.runtime_api import LDS_READ_OPS, lds_read_cost
+    b32, b64 = LDS_READ_OPS.index("ds_read_b32"), LDS_READ_OPS.index("ds_read_b64")
+    linear, scattered = lds_read_cost(b64, 0, 0), lds_read_cost(b64, 1, 0)
+    assert 1.0 < linear < 6.0 and linear < scattered < 30.0                # bank conflicts cost cycles
+    assert abs(lds_read_cost(b32, 0, 0) - linear) < 1.0                    # 4 and 8 bytes per lane cost the same
+    with pytest.raises(RuntimeError):
+        lds_read_cost(b32, 3, 0)
 
 
 @pytest.mark.parametrize("k,rows", [(2, 20000), (3, 9000), (1, 777)])

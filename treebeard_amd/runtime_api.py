@@ -118,6 +118,26 @@ def lds_read_bandwidth(width_bytes):
     return rate.value
 
 
+LDS_READ_OPS = ("ds_read_b32", "ds_read_b64", "ds_read_b128", "ds_read2_b32", "ds_read_u16", "ds_read_u8", "ds_read_b96")
+
+
+def lds_read_cost(op, pattern=0, mask=0):
+    """Cycles (nominal shader clock) a compute unit spends per wave-level LDS read, measured by the bench-only
+    library.  op indexes LDS_READ_OPS; pattern 0 = lane i reads element i, 1 = random over 48 KB, 2 = random over
+    1 KB, 5..7 = random among 2**pattern consecutive elements; mask 0 = all lanes, 1 = lanes 0-31, 2 = even lanes,
+    3 = a random half, 4 = a random quarter."""
+    if not os.path.exists(BENCH_LIB_PATH):
+        raise FileNotFoundError("%s is missing: build it with `python -m treebeard_amd.build`" % BENCH_LIB_PATH)
+    lib = ctypes.CDLL(BENCH_LIB_PATH)
+    lib.tbbench_lds_read_cost.restype = c_i32
+    lib.tbbench_lds_read_cost.argtypes = [c_i32, c_i32, c_i32, ctypes.POINTER(ctypes.c_double)]
+    cycles = ctypes.c_double()
+    rc = lib.tbbench_lds_read_cost(op, pattern, mask, ctypes.byref(cycles))
+    if rc != 0:
+        raise RuntimeError("LDS read-cost measurement failed with HIP error %d" % rc)
+    return cycles.value
+
+
 _api = None
 
 
