@@ -2,9 +2,10 @@
 
 Bars: per-tree leaf selection bit-exact; predictions within 1e-5 relative of the
 oracle (sums) and 1e-6 absolute (sigmoid / softmax); class ids equal.  At the
-full benchmark sizes, where the oracle would take minutes, the checks are
-size-independent properties (sub-batch consistency, permutation equivariance)
-plus an oracle comparison on a random sample of rows.
+full benchmark sizes the whole batch is compared with the oracle when the host
+has at least 8 threads to split the rows over (a random sample of rows
+otherwise), next to size-independent properties (sub-batch consistency,
+permutation equivariance).
 """
 import ctypes
 import os
@@ -198,9 +199,11 @@ def test_full_size_properties(synth_model, k):
     full = gpu_predict(runner, x)
     assert not np.isnan(full.astype(np.float32)).any()
     rng = np.random.default_rng(k)
-    # (1) a random sample of rows against the oracle
-    pick = rng.choice(rows, size=4096, replace=False)
-    pred, _ = cpu_oracle.predict(forest, x[pick])
+    # (1) every row against the oracle when the host has the cores to walk the whole batch in seconds
+    # (rows split over the threads), else a random sample of rows
+    threads = cpu_oracle.max_threads()
+    pick = slice(None) if threads >= 8 else rng.choice(rows, size=4096, replace=False)
+    pred, _ = cpu_oracle.predict(forest, x if threads >= 8 else x[pick], threads=threads)
     if forest.num_classes > 0:
         np.testing.assert_array_equal(full[pick].astype(np.float32), pred)
     elif forest.transform == model_io.SIGMOID:
