@@ -252,6 +252,9 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
     __syncthreads();
     if (g + 1 < gEnd) TBAMD_PREFETCH_GROUP(groups[g + 1]) // in flight while this group is walked
 
+    // Walking waves go before waves that are staging (this block's or the other block's on the CU): the walk is
+    // what keeps the LDS and the VALUs busy.
+    __builtin_amdgcn_s_setprio(1);
     // Bundles are sorted by class; a segment is a run of bundles of one class.
     uint32_t b0 = 0;
     while (b0 < grp.bundleCount) {
@@ -331,6 +334,7 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
       }
       b0 = b1;
     }
+    __builtin_amdgcn_s_setprio(0);
   }
 
   if (C > 0) {
