@@ -170,6 +170,11 @@ TBAMD_EXPORT int32_t tbmi_set_global_walk_plan(intptr_t runner, int32_t rowsPerB
 /* Pins the row-parallel kernel on rank-quantised rows (64 rows per block, one byte per feature value). */
 TBAMD_EXPORT int32_t tbmi_set_quantized_plan(intptr_t runner, int32_t treeThreads, int32_t interleave,
                                              int32_t groupBytes, int32_t treeSlices);
+/* How the row-parallel scalar walk brings tree groups into LDS: 0 by rule (direct global-to-LDS copies when two
+ * blocks fit a compute unit, through prefetch registers otherwise), 1 always through registers, 2 always direct.
+ * Results do not depend on it.  No counterpart in the reference (its GPU schedules cache trees with cooperative
+ * loads, src/gpu/GPURepresentations.cpp:279-399). */
+TBAMD_EXPORT int32_t tbmi_set_group_staging(intptr_t runner, int32_t mode);
 TBAMD_EXPORT int32_t tbmi_describe_plan(intptr_t runner, char *buffer, int32_t length);
 /* Compile once, reload: saves the compiled model (forest + launch plan) of a runner to one file and
  * reopens it without the source model (batchSize <= 0 keeps the saved batch size).  Stands in for

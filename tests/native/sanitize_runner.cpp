@@ -281,7 +281,14 @@ void DeviceEntryPoints(const Case &c, int64_t rows, int32_t tileSize = 1, int32_
   const int rowsLds[][5] = {{64, 1, 1, 16384, 1}, {128, 1, 2, 32768, 3}, {256, 1, 8, 65536, 1}, {512, 1, 4, 49152, 5}, {256, 1, 4, 8192, 40},
                             {256, 4, 4, 65536, 1}, {128, 8, 2, 40960, 2}, {64, 3, 1, 16384, 1}, {512, 2, 8, 32768, 1}};
   for (auto &p : rowsLds)
-    if (tbmi_set_plan(runner, p[0], p[1], p[2], p[3], p[4]) == 0) runAll("rows_lds plan");
+    if (tbmi_set_plan(runner, p[0], p[1], p[2], p[3], p[4]) == 0) {
+      runAll("rows_lds plan");
+      for (int mode : {1, 2, 0}) { // tree groups through registers, copied directly, by rule
+        EXPECT(tbmi_set_group_staging(runner, mode) == 0, "tbmi_set_group_staging");
+        runAll("rows_lds plan, group staging pinned");
+      }
+    }
+  EXPECT(tbmi_set_group_staging(runner, 7) != 0, "tbmi_set_group_staging refuses an unknown mode");
   const int treeParallel[][5] = {{1, 256, 1, 0, 0}, {4, 64, 1, 32768, 7}, {16, 16, 2, 0, 1}, {2, 128, 1, 16384, 0}, {8, 8, 4, 0, 3}, {64, 1, 1, 0, 2}, {1, 1024, 1, 65536, 1}};
   for (auto &p : treeParallel)
     if (tbmi_set_tree_parallel_plan(runner, p[0], p[1], p[2], p[3], p[4]) == 0) runAll("tree_parallel plan");

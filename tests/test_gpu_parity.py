@@ -233,7 +233,38 @@ def test_launch_plans_agree(synth_model, k, plan):
     runner = make_runner(synth_model(k), 3001)
     runner.set_plan(*plan)
     assert "kernel=rows_lds rowsPerBlock=%d treeThreads=%d treeLanes=1 interleave=%d" % plan[:3] in runner.describe_plan()
-    check_against_oracle(runner, forest, x)
+    # both ways of bringing tree groups into LDS: through prefetch registers, and by direct global-to-LDS copies
+    results = []
+    for mode, name in ((1, "registers"), (2, "direct")):
+        runner.set_group_staging(mode)
+        assert "staging=" + name in runner.describe_plan()
+        results.append(check_against_oracle(runner, forest, x))
+    np.testing.assert_array_equal(results[0], results[1])
+
+
+@pytest.mark.parametrize("k", [1, 2, 3, 4, 5])
+def test_group_staging_follows_the_blocks_per_compute_unit(synth_model, k):
+    """By rule tree groups are copied straight into LDS when two blocks fit a compute unit (one walks while the
+    other waits for its copy) and go through prefetch registers otherwise; either way the results are the same."""
+    cfg = synth.CONFIGS[k]
+    rows = 1 << 16 if k != 4 else 1 << 12       # (enough row blocks for one tree slice)
+    forest = model_io.load_xgboost_json(synth_model(k))
+    x = cfg.batch_rows(rows, seed_offset=21)
+    runner = make_runner(synth_model(k), rows)
+    plan = runner.describe_plan()
+    if "kernel=rows_lds" not in plan:
+        pytest.skip("the automatic plan for this batch is not the row-parallel kernel: " + plan)
+    lds = int(plan.split("ldsBytes=")[1].split()[0])
+    assert ("staging=direct" in plan) == (2 * (lds + 512) <= 160 * 1024), plan
+    by_rule = gpu_predict(runner, x)
+    for mode in (1, 2):
+        runner.set_group_staging(mode)
+        np.testing.assert_array_equal(gpu_predict(runner, x), by_rule)
+    runner.set_group_staging(0)
+    sample = slice(0, 2048)
+    np.testing.assert_array_equal(gpu_leaf_ids(runner, x[sample]), cpu_oracle.leaf_ids(forest, x[sample]))
+    with pytest.raises(RuntimeError):
+        runner.set_group_staging(3)
 
 
 @pytest.mark.parametrize("plan", [(1, 256, 1, 0, 0), (4, 64, 1, 32768, 7), (16, 16, 2, 0, 1), (2, 128, 1, 16384, 0),

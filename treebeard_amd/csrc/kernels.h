@@ -36,6 +36,9 @@ struct WalkParams {
   const DeviceGlobalNode *globalNodes = nullptr; // global-memory walk only
   const DeviceGlobalTree *globalTrees = nullptr;
   bool peelWalks = false;         // bundles carry peel depths below their depths: use the kernels that look at them
+  // Row-parallel scalar walk: tree groups go straight from global memory into LDS (no staging registers); the
+  // block waits for its copy, so this pays when a second block on the CU walks meanwhile.
+  bool directStaging = false;
   float *out = nullptr;           // used when the epilogue is fused (1 slice; class ids as float32 with fuseArgmax)
   int8_t *classOut = nullptr;     // fuseArgmax: class ids as int8 (out is then null)
   double *partial = nullptr;      // [partials][rows][max(1, classes)] otherwise

@@ -196,8 +196,9 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
   int bestClass = 0;
 
   // Register double buffer for the next tree group.  Loads are unconditional
-  // (index clamped) so that they stay in flight across the walk.
-  U32x4 fetched[PF];
+  // (index clamped) so that they stay in flight across the walk.  PF == 0 is the other way of staging: no
+  // registers, the group goes straight from global memory into LDS between the two barriers (below).
+  U32x4 fetched[PF > 0 ? PF : 1];
 #define TBAMD_PREFETCH_GROUP(NEXTGRP)                                                                                  \
   {                                                                                                                    \
     const DeviceGroup nextGrp = (NEXTGRP);                                                                             \
@@ -235,12 +236,12 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
     }                                                                                                                  \
     acc = 0.0;                                                                                                         \
   }
-  if (gBegin < gEnd) TBAMD_PREFETCH_GROUP(groups[gBegin])
+  if (PF > 0 && gBegin < gEnd) TBAMD_PREFETCH_GROUP(groups[gBegin])
 
   for (int g = gBegin; g < gEnd; ++g) {
     const DeviceGroup grp = groups[g];
     __syncthreads(); // rows staged / previous group no longer read
-    {
+    if (PF > 0) {
       U32x4 *dst = reinterpret_cast<U32x4 *>(lds);
       const int pieces = (int)(grp.nodeCount >> 1);
 #pragma unroll
@@ -248,9 +249,22 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
         const int idx = tid + i * threads;
         if (idx < pieces) dst[idx] = fetched[i];
       }
+    } else {
+      // Direct staging: the group is copied by global -> LDS loads (lane i of a wave-wide load leaves its 16 bytes
+      // at base + 16 i, lanes switched off write nothing): no staging registers, no LDS store instructions.  The
+      // block waits for its own copy; the CU's other block walks meanwhile, which is why launch plans ask for
+      // this form only when two blocks fit a CU.
+      const U32x4 *src = reinterpret_cast<const U32x4 *>(nodes16) + (grp.nodeBegin >> 1);
+      const int pieces = (int)(grp.nodeCount >> 1);
+      const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+      for (int first = wave * 64; first < pieces; first += threads)
+        if (first + (tid & 63) < pieces)
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + first + (tid & 63)),
+                                           (__attribute__((address_space(3))) void *)(lds + (uint32_t)first * 16u), 16, 0, 0);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     __syncthreads();
-    if (g + 1 < gEnd) TBAMD_PREFETCH_GROUP(groups[g + 1]) // in flight while this group is walked
+    if (PF > 0 && g + 1 < gEnd) TBAMD_PREFETCH_GROUP(groups[g + 1]) // in flight while this group is walked
 
     // Walking waves go before waves that are staging (this block's or the other block's on the CU): the walk is
     // what keeps the LDS and the VALUs busy.
@@ -1053,6 +1067,7 @@ hipError_t LaunchWalkKP(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBy
 
 template <int K, int W>
 hipError_t LaunchWalkK(const WalkParams &p, int prefetch, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
+  if (p.directStaging) return LaunchWalkKP<K, 0, W>(p, grid, block, ldsBytes, stream);
   if (prefetch <= 4) return LaunchWalkKP<K, 4, W>(p, grid, block, ldsBytes, stream);
   if (prefetch <= 8) return LaunchWalkKP<K, 8, W>(p, grid, block, ldsBytes, stream);
   if (prefetch <= 16) return LaunchWalkKP<K, 16, W>(p, grid, block, ldsBytes, stream);

@@ -242,6 +242,20 @@ void InferenceRunner::EnsureStaging(int64_t rows) {
   m_stageRows = rows;
 }
 
+void InferenceRunner::SetGroupStaging(int32_t mode) {
+  if (mode < 0 || mode > 2) throw Error("group staging mode must be 0 (by rule), 1 (registers) or 2 (direct)");
+  m_groupStaging = mode;
+}
+
+bool InferenceRunner::DirectStaging() const {
+  const LaunchPlan &plan = m_model.plan;
+  if (plan.kernel != LaunchPlan::Kernel::kRowParallelLds || plan.tileSize > 1) return false; // (only the scalar row-parallel walk has the form)
+  if (m_groupStaging != 0) return m_groupStaging == 2;
+  // Measured on MI355X (28 to 520 features, 600 to 1000 trees): 5 to 15 % faster with two blocks per CU,
+  // 2 to 4 % slower with one, whose wait for the copy nothing covers.  (LDS is handed out in coarse pieces.)
+  return 2 * (m_model.LdsBytes() + 512) <= (size_t)m_limits.ldsBytesPerBlock;
+}
+
 hipError_t InferenceRunner::LaunchWalk(const WalkParams &p, hipStream_t stream) const {
   const LaunchPlan &plan = m_model.plan;
   if (plan.kernel == LaunchPlan::Kernel::kGlobalWalk) return LaunchWalkGlobal(p, plan.interleave, stream);
@@ -267,6 +281,7 @@ WalkParams InferenceRunner::MakeWalkParams(const float *deviceInputs, int64_t ro
   p.s.treeLanes = m_model.plan.treeLanes;
   p.s.initialValue = m_forest.initialValue;
   p.peelWalks = m_model.plan.peelWalks;
+  p.directStaging = DirectStaging();
   p.x = deviceInputs;
   p.globalNodes = m_dGlobalNodes;
   p.globalTrees = m_dGlobalTrees;
@@ -576,6 +591,7 @@ std::string InferenceRunner::DescribePlan() const {
      << " groups=" << m_model.groups.size()
      << " bundles=" << m_model.bundles.size() << " nodes=" << m_model.nodes.size()
      << " ldsBytes=" << m_model.LdsBytes() << " tileSize=" << p.tileSize << " tiling=" << p.tiling
+     << " staging=" << (DirectStaging() ? "direct" : "registers")
      << " peelWalks=" << (p.peelWalks ? 1 : 0) << " treesTiledByProfile=" << m_model.treesTiledByProfile
      << " lockStepSteps=" << m_model.lockStepSteps << " profiledSteps=" << m_model.profiledSteps;
   return os.str();

@@ -82,6 +82,11 @@ public:
   int32_t ReturnTypeBytes() const { return ClassIdsAsInt8() ? 1 : 4; }
   const CompilerOptions &Options() const { return m_options; }
   int64_t LastKernelMicros() const { return m_lastKernelMicros; }
+  // How the row-parallel scalar walk brings tree groups into LDS: 0 by rule (direct global -> LDS copies when two
+  // blocks fit a CU, so that one walks while the other waits for its copy; through prefetch registers
+  // otherwise), 1 always through registers, 2 always direct.
+  void SetGroupStaging(int32_t mode);
+  bool DirectStaging() const;
   const PackedModel &Model() const { return m_model; }
   const Forest &GetForest() const { return m_forest; }
   const HitCountProfile *Profile() const { return m_profile.get(); }
@@ -151,6 +156,7 @@ private:
   void *m_dStageOut = nullptr;
   int64_t m_stageRows = 0;
   int64_t m_lastKernelMicros = 0;
+  int32_t m_groupStaging = 0;
 };
 
 } // namespace tbamd

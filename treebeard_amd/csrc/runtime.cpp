@@ -447,6 +447,15 @@ int32_t tbmi_set_quantized_plan(intptr_t h, int32_t treeThreads, int32_t interle
       -1);
 }
 
+int32_t tbmi_set_group_staging(intptr_t h, int32_t mode) {
+  return Guard(
+      [&] {
+        Runner(h)->SetGroupStaging(mode);
+        return 0;
+      },
+      -1);
+}
+
 int32_t tbmi_describe_plan(intptr_t h, char *buffer, int32_t length) {
   return Guard(
       [&] {
