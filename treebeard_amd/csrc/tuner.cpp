@@ -317,9 +317,9 @@ std::vector<LaunchPlan> CandidatePlans(const Forest &forest, int64_t batchSize, 
   }
   const int64_t need = (BiggestTreeNodes(forest) + 2) * kNodeBytes;
   for (int32_t rb : {64, 128, 256, 512})
-    for (int32_t tt : {1, 2, 4, 8})
+    for (int32_t tt : {1, 2, 4, 8, 16})
       for (int32_t k : {2, 4, 8})
-        for (int blocksPerCu : {1, 2, 3}) {
+        for (int blocksPerCu : {1, 2, 3, 4}) {
           if (rb * tt > 1024) continue;
           bool words = false;
           const int32_t budget = limits.ldsBytesPerBlock / blocksPerCu;
