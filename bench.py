@@ -179,8 +179,8 @@ def main():
                 "algorithmic_bytes_per_row": lds_bytes_row, "visited_nodes_per_row": steps_per_row,
                 "measured_lds_read_gbs": lds_measured, "lds_floor": lds_floor,
                 "frac_of_measured_lds": (lds_gbs / lds_measured["b128"]) if lds_measured else None,
-                "peak_note": "256 CUs x 256 B/clk x 2.4 GHz; a scalar walk moves 10 B per lane per two LDS "
-                             "instructions of 2 clk each, so 62.5 % is its ceiling"}
+                "peak_note": "256 CUs x 256 B/clk x 2.4 GHz; a scalar walk moves 10 B per lane in two LDS "
+                             "instructions of about 2.5 clk each (measured), so about 50 % is its ceiling"}
     roofline = dict(lds_view if binding == "lds" else hbm_view)
     roofline.update({"traffic": traffic, "traffic_source": "profiles/hbm_traffic.json (rocprofv3 FETCH_SIZE + WRITE_SIZE "
                                                            "of this command, scaled by a plain copy)" if traffic else None,
