@@ -767,6 +767,7 @@ def test_random_forests_and_plans(tmp_path, seed):
                                                          num_tree_threads=int(rng.choice([1, 2, 4, 10])))
         gpu.TreeWalkInterleaveFactor(int(rng.choice([1, 2, 4, 8])))
     runner = make_runner(path, rows, gpu_options=gpu)
+    runner.set_group_staging(int(rng.integers(0, 3)))     # tree groups by rule, through registers, or copied directly
     check_against_oracle(runner, forest, x)
     kind = rng.integers(0, 4)
     try:
