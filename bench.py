@@ -53,6 +53,8 @@ def main():
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (default: the headline, 2)")
     ap.add_argument("--rows", type=int, default=0, help="override the batch size")
     ap.add_argument("--tile-size", type=int, default=1, help="CompilerOptions tile size (2, 3, 4 run the tiled walk kernel)")
+    ap.add_argument("--group-staging", type=int, default=0, choices=[0, 1, 2],
+                    help="how tree groups reach LDS: 0 by rule, 1 through prefetch registers, 2 direct global-to-LDS copies")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--autotune", action="store_true", help="timed launch-plan search before measuring")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU-baseline duration")
@@ -81,6 +83,8 @@ def main():
         options.SetReturnTypeWidth(8)
         options.SetReturnTypeIsFloatType(False)
     runner = treebeard.TreebeardInferenceRunner.FromModelFile(model, "", options)
+    if args.group_staging:
+        runner.set_group_staging(args.group_staging)
     multiclass = runner.num_classes() > 0
     dx = torch.from_numpy(x).cuda()
     out = torch.zeros(rows, dtype=torch.int8 if multiclass else torch.float32, device="cuda")
