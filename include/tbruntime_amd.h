@@ -120,9 +120,14 @@ TBAMD_EXPORT int32_t tbmi_device_count(void);
 TBAMD_EXPORT int32_t tbmi_run_device(intptr_t runner, const float *deviceInputs, void *deviceResults, int64_t rows);
 /* The same kernels enqueued on the caller's stream (a hipStream_t; null is the default stream); the call
  * returns without waiting for them.  Work queued on that stream before the call is seen by the kernels,
- * work queued after it sees their results: no synchronisation is needed on either side.  The first call,
- * and a call with more rows than any before it, allocates the runner's partial-sum buffers; while such a
- * call is made no earlier call on another stream may still be running. */
+ * work queued after it sees their results: no synchronisation is needed on either side.  All calls on one
+ * runner share its device buffers (the packed model, partial sums, rank-quantised rows); the library records
+ * an event behind the kernels of every call made here, and the next call on this runner - on another stream,
+ * or through an entry point that uses the runner's own stream - waits for it on the device, while calls that
+ * re-pack the model (tbmi_set_*_plan, tbmi_autotune), grow the buffers (the first call, and a call with more
+ * rows than any before it, allocates) or delete the runner wait for it on the host.  Calls on one runner are
+ * therefore ordered, never concurrent; use one runner per stream for kernels that should overlap.  One caller
+ * thread per runner, as in the reference. */
 TBAMD_EXPORT int32_t tbmi_run_device_async(intptr_t runner, const float *deviceInputs, void *deviceResults,
                                            int64_t rows, void *stream);
 /* No counterpart in the reference.  For callers that cannot allocate device memory (code under HIP graph
@@ -132,7 +137,10 @@ TBAMD_EXPORT int32_t tbmi_run_device_async(intptr_t runner, const float *deviceI
  * bytes (32 MiB) that the library holds on every GPU it runs on.  It allocates, frees and synchronises
  * nothing.  A call whose plan needs more scratch memory than that for `rows` rows fails with a message
  * naming both sizes (pass fewer rows per call).  All calls on one GPU share the array: calls that overlap
- * in time on one GPU, from any runner or stream, race on it. */
+ * in time on one GPU, from any runner or stream, race on it.  Because it may be captured into a graph this
+ * entry point records no event either: the caller keeps the runner alive and un-repacked (no tbmi_set_*_plan,
+ * tbmi_autotune, DeleteInferenceRunner) until the kernels of its calls have finished.  The array costs every
+ * process that loads the library 32 MiB of device memory per GPU it touches. */
 TBAMD_EXPORT int32_t tbmi_run_device_noalloc(intptr_t runner, const float *deviceInputs, void *deviceResults,
                                              int64_t rows, void *stream);
 TBAMD_EXPORT int64_t tbmi_noalloc_scratch_bytes(void);
@@ -181,6 +189,12 @@ TBAMD_EXPORT int32_t tbmi_describe_plan(intptr_t runner, char *buffer, int32_t l
  * InitializeInferenceRunner(soPath, globalsJSON), runtime.cpp:35-54. */
 TBAMD_EXPORT int32_t tbmi_save_compiled_model(intptr_t runner, const char *path);
 TBAMD_EXPORT intptr_t tbmi_load_compiled_model(const char *path, int32_t batchSize);
+/* src/runtime/runtime.cpp:35-54 (`InitializeInferenceRunner(soPath, modelGlobalsJSONPath)`, bound by
+ * src/python/treebeard.py:314-319 FromSOFile): reopens a compiled model with the saved batch size.  `soPath` names
+ * a file written by tbmi_save_compiled_model, which also holds what the reference keeps in its model-globals
+ * JSON (tile size, type widths, the model buffers' contents); `modelGlobalsJSONPath` is accepted and not opened.
+ * Returns 0 on failure (message in tbmi_last_error). */
+TBAMD_EXPORT intptr_t InitializeInferenceRunner(const char *soPath, const char *modelGlobalsJSONPath);
 TBAMD_EXPORT int32_t tbmi_num_trees(intptr_t runner);
 TBAMD_EXPORT int32_t tbmi_num_classes(intptr_t runner);
 

@@ -251,6 +251,25 @@ uint32_t TileStepHost(const unsigned char *group, uint32_t groupBytes, uint32_t 
   const uint32_t bytes = TileBytes(T);
   if (addr % 8 != 0 || addr + bytes > groupBytes) std::abort(); // tile outside the group
   const unsigned char *tile = group + addr;
+  if (T > kMaxSelectTile) { // the eight-slot tile: { thr[8]; off[8]; links; childBase }
+    float thr8[8];
+    uint16_t off8[8], base;
+    uint64_t links;
+    std::memcpy(thr8, tile, 32);
+    std::memcpy(off8, tile + 32, 16);
+    std::memcpy(&links, tile + 48, 8);
+    std::memcpy(&base, tile + 56, 2);
+    uint32_t slot = 0;
+    for (int hop = 0; hop < 8; ++hop) {
+      if (off8[slot] % stride != 0 || (int)(off8[slot] / stride) > F) std::abort();
+      const int f = (int)(off8[slot] / stride);
+      const float x = f == F ? -INFINITY : row[f];
+      const uint32_t link = (uint32_t)(links >> (8 * slot + (x < thr8[slot] ? 4 : 0))) & 15u;
+      if (link >= kTileLinkExit) return base + (link - kTileLinkExit) * bytes;
+      slot = link + 1;
+    }
+    std::abort(); // links that never reach a child
+  }
   float thr[kMaxTileSize];
   uint16_t off[kMaxTileSize], childBase;
   std::memcpy(thr, tile, (size_t)T * 4);
@@ -288,8 +307,7 @@ hipError_t LaunchWalkRowsTiled(const WalkParams &p, int tileSize, int interleave
   if (ldsBytes > 160 * 1024 || RB < 64 || (RB & (RB - 1)) || TT < 1 || RB * TT > 1024) return hipErrorInvalidValue;
   if ((int64_t)(p.s.numFeatures + 1) * RB * 4 > 0x10000) return hipErrorInvalidValue;
   if (p.s.treeSlices < 1 || p.s.treeSlices > 65535) return hipErrorInvalidValue;
-  if ((int)((p.s.groupRegionBytes / 16 + RB * TT - 1) / (RB * TT)) > 16) return hipErrorInvalidValue;
-  if (T < 2 || T > 4 || (K != 1 && K != 2 && K != 4)) return hipErrorInvalidValue;
+  if (T < 2 || T > kMaxTileSize || (K != 1 && K != 2 && K != 4)) return hipErrorInvalidValue;
   if (p.s.treeSlices > 1 && !p.partial) std::abort();
   const DeviceNode *nodes = reinterpret_cast<const DeviceNode *>(p.nodes16);
   const int F = p.s.numFeatures;

@@ -249,7 +249,7 @@ void DeviceEntryPoints(const Case &c, int64_t rows, int32_t tileSize = 1, int32_
   };
   runAll("default plan");
   if (tileSize > 1) { // block shapes of the tiled walk, the plan search, save and reload
-    const int tiledPlans[][5] = {{64, 1, 1, 16384, 1}, {128, 8, 2, 32768, 3}, {256, 4, 4, 40960, 2}, {64, 16, 2, 24576, 5}};
+    const int tiledPlans[][5] = {{64, 1, 1, 16384, 1}, {128, 8, 2, 32768, 3}, {256, 4, 4, 40960, 2}, {64, 16, 2, 24576, 5}, {128, 4, 1, 65536, 2}};
     for (auto &p : tiledPlans)
       if (tbmi_set_plan(runner, p[0], p[1], p[2], p[3], p[4]) == 0) runAll("tiled plan");
     EXPECT(tbmi_set_tree_parallel_plan(runner, 4, 64, 1, 0, 1) == -1, "tree-parallel plan must refuse tiles");
@@ -348,7 +348,7 @@ int main(int argc, char **argv) {
     if (!Quick()) {
       const std::string profile =
           WriteProfile(c, std::string(std::getenv("TMPDIR") ? std::getenv("TMPDIR") : "/tmp") + "/sanitize_profile.csv");
-      for (int32_t tileSize : {2, 3, 4}) {
+      for (int32_t tileSize : {2, 3, 4, 5, 8}) {
         DeviceEntryPoints(c, std::min<int64_t>(c.rows, 203), tileSize);
         DeviceEntryPoints(c, std::min<int64_t>(c.rows, 203), tileSize, 1, profile.c_str(), true);
         DeviceEntryPoints(c, std::min<int64_t>(c.rows, 203), tileSize, 2, profile.c_str(), false);
@@ -356,9 +356,9 @@ int main(int argc, char **argv) {
       DeviceEntryPoints(c, std::min<int64_t>(c.rows, 203), 1, 1, profile.c_str(), true); // scalar nodes, peeled walks
       const intptr_t options = CreateCompilerOptions();
       Set_batchSize(options, 64);
-      Set_tileSize(options, 8);
-      EXPECT(CreateInferenceRunner(c.path.c_str(), "", options) == 0 && std::strstr(tbmi_last_error(), "tile size 8"),
-             "tile size 8 must be refused");
+      Set_tileSize(options, 9);
+      EXPECT(CreateInferenceRunner(c.path.c_str(), "", options) == 0 && std::strstr(tbmi_last_error(), "tile size 9"),
+             "tile size 9 must be refused");
       DeleteCompilerOptions(options);
     }
     std::printf("%s: %lld rows done, %d failures so far\n", argv[a], (long long)c.rows, gFailures);

@@ -50,7 +50,8 @@ def _attr(name, ints=None, floats=None, strings=None, s=None, i=None, packed=Fal
 def write_onnx(path, trees, mode="BRANCH_LT", base_value=0.0, post_transform="NONE", classifier=False,
                n_classes=0, class_ids=None, packed=False):
     """trees: list of (value, feature, left, right) with local child indices (-1 on leaves); node ids
-    are the local indices, the true branch is `left`."""
+    are the local indices, the true branch is `left`.  class_ids[t] is the class tree t votes for, or a
+    sequence that gives every leaf of tree t (in node order) a class id of its own."""
     tree_ids, node_ids, feats, vals, true_ids, false_ids, modes = [], [], [], [], [], [], []
     t_tree, t_node, t_ids, t_w = [], [], [], []
     for t, (value, feature, left, right) in enumerate(trees):
@@ -63,8 +64,11 @@ def write_onnx(path, trees, mode="BRANCH_LT", base_value=0.0, post_transform="NO
             false_ids.append(0 if leaf else int(right[n]))
             modes.append("LEAF" if leaf else mode)
             if leaf:
+                cls = class_ids[t] if class_ids is not None else 0
+                if hasattr(cls, "__len__"):
+                    cls = cls[len([m for m in t_tree if m == t]) % len(cls)]
                 t_tree.append(t); t_node.append(n)
-                t_ids.append(int(class_ids[t]) if class_ids is not None else 0)
+                t_ids.append(int(cls))
                 t_w.append(float(value[n]))
     node = _bytes_field(4, b"TreeEnsembleClassifier" if classifier else b"TreeEnsembleRegressor")
     node += _attr("base_values", floats=[base_value], packed=packed)

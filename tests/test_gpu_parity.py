@@ -154,6 +154,51 @@ def test_onnx_comparison_modes(tmp_path, mode):
     check_against_oracle(runner, forest, x)
 
 
+@pytest.mark.parametrize("slices", [1, 2])
+@pytest.mark.parametrize("post_transform", ["NONE", "LOGISTIC", "SOFTMAX"])
+def test_onnx_classifier(tmp_path, post_transform, slices):
+    """TreeEnsembleClassifier through the ONNX loader (src/json/onnxmodelparser.h:102-113, :162-172, :355-374):
+    one class id per tree, any post_transform; leaf ids and class ids against the oracle on the forest its own
+    loader reads, with leaf weights on a coarse grid so that class sums tie exactly on many rows (the larger
+    class id wins, src/reduction/LowerReduceOps.cpp:148-187), on the walk kernel's own arg-max (one tree slice)
+    and through the finalize kernel (two)."""
+    rng = np.random.Generator(np.random.PCG64(77))
+    classes, features = 6, 5
+    split = lambda: (rng.integers(0, features), rng.normal())
+    grown = [synth._grow_tree(rng, 4, lambda d, s: 0.8, split, lambda: float(rng.integers(-2, 3)) * 0.25) for _ in range(40)]
+    trees = [(np.asarray(t.value, np.float32), t.feature, t.left, t.right) for t in grown]
+    class_ids = [int(c) for c in rng.integers(0, classes - 1, len(trees))]           # the last class gets no tree
+    path = tmp_path / "classifier.onnx"
+    write_onnx(path, trees, base_value=0.25, post_transform=post_transform, classifier=True, n_classes=classes, class_ids=class_ids)
+    forest = model_io.load_onnx(path, features)
+    assert forest.num_classes == classes and list(forest.class_id) == class_ids
+    rows = 1500
+    x = rng.normal(size=(rows, features)).astype(np.float32)
+    runner = make_runner(path, rows, "onnx_file", features)
+    assert runner.result_dtype() == np.int8
+    runner.set_plan(64, 2, 2, 4096, slices)
+    got = check_against_oracle(runner, forest, x)
+    _, sums = cpu_oracle.predict(forest, x)
+    best = sums.max(axis=1, keepdims=True)
+    assert ((sums == best).sum(axis=1) > 1).sum() > 20          # exact ties for the maximum do occur
+    ties = (sums[:, :classes - 1] == best).sum(axis=1) > 1
+    voted = np.where(sums[:, :classes - 1] == best, np.arange(classes - 1)[None, :], -1).max(axis=1)
+    unvoted_wins = 0.25 >= best[:, 0]                           # the class without trees scores the base value
+    np.testing.assert_array_equal(got[ties & ~unvoted_wins], voted[ties & ~unvoted_wins])
+
+
+def test_onnx_classifier_with_several_class_ids_in_one_tree_is_refused(tmp_path):
+    rng = np.random.Generator(np.random.PCG64(78))
+    grown = [synth._grow_tree(rng, 3, lambda d, s: 0.9, lambda: (rng.integers(0, 3), rng.normal()), lambda: rng.normal()) for _ in range(3)]
+    trees = [(np.asarray(t.value, np.float32), t.feature, t.left, t.right) for t in grown]
+    path = tmp_path / "mixed.onnx"
+    write_onnx(path, trees, classifier=True, n_classes=3, class_ids=[0, [1, 2], 2])
+    options = treebeard.CompilerOptions(64, 1)
+    options.SetNumberOfFeatures(3)
+    with pytest.raises(RuntimeError, match="multiple class IDs per tree"):
+        treebeard.TreebeardInferenceRunner.FromONNXModelFile(str(path), options)
+
+
 # --------------------------------------------------------------------------
 # the benchmark configurations at oracle-sized batches
 # --------------------------------------------------------------------------
@@ -464,6 +509,13 @@ def test_compiled_model_file_round_trip(synth_model, tmp_path, k):
     np.testing.assert_array_equal(gpu_predict(reopened, x), expected)
     forest = model_io.load_xgboost_json(synth_model(k))
     np.testing.assert_array_equal(gpu_leaf_ids(reopened, x[:256]), cpu_oracle.leaf_ids(forest, x[:256]))
+    # the reference's own entry point for reopening a compiled model (src/runtime/runtime.cpp:35-54, FromSOFile)
+    again = treebeard.TreebeardInferenceRunner.FromSOFile(path, str(tmp_path / "globals.json"))
+    assert again.batchSize == rows and again.rowSize == forest.num_features and again.describe_plan() == plan
+    check_against_oracle(again, forest, x)
+    np.testing.assert_array_equal(again.RunInference(x), expected)
+    with pytest.raises(RuntimeError, match="InitializeInferenceRunner"):
+        treebeard.TreebeardInferenceRunner.FromSOFile(str(tmp_path / "missing.tbamd"), "")
     with open(path, "r+b") as fh:
         fh.truncate(os.path.getsize(path) // 2)
     with pytest.raises(RuntimeError, match="truncated"):
@@ -830,7 +882,7 @@ def test_async_entry_point_orders_itself_on_the_callers_stream(synth_model, k, r
 
 
 # --------------------------------------------------------------------------
-# tiled walks (CompilerOptions tile size 2, 3, 4) and probability-based tiling
+# tiled walks (CompilerOptions tile size 2 to 8) and probability-based tiling
 # --------------------------------------------------------------------------
 def make_tiled_runner(path, batch, tile_size, tiling_type=0, profile="", peel=False, multiclass=False):
     options = treebeard.CompilerOptions(batch, tile_size)
@@ -859,7 +911,7 @@ def write_profile(path, forest, ids):
     return str(path)
 
 
-@pytest.mark.parametrize("tile_size", [2, 3, 4])
+@pytest.mark.parametrize("tile_size", [2, 3, 4, 5, 7, 8])
 @pytest.mark.parametrize("k,rows", [(1, 1024), (2, 4096), (3, 4096), (5, 2048)])
 def test_tiled_walk_selects_the_scalar_walks_leaves(synth_model, k, rows, tile_size):
     """Set_tileSize > 1 runs the tiled kernel; its leaves are those of the scalar oracle and of the tiled CPU walk."""
@@ -873,7 +925,7 @@ def test_tiled_walk_selects_the_scalar_walks_leaves(synth_model, k, rows, tile_s
     check_against_oracle(runner, forest, x)
 
 
-@pytest.mark.parametrize("tile_size", [2, 4])
+@pytest.mark.parametrize("tile_size", [2, 4, 8])
 def test_tiled_walk_on_the_reference_fixtures(plain_file, tile_size):
     for name in BENCHMARK_XGB:
         path = plain_file(benchmark_model(name))
@@ -892,7 +944,7 @@ def test_tiled_walk_on_the_reference_fixtures(plain_file, tile_size):
 
 
 @pytest.mark.parametrize("plan", [(64, 1, 1, 16384, 1), (128, 8, 2, 32768, 3), (256, 4, 4, 40960, 2), (64, 16, 2, 24576, 5)])
-@pytest.mark.parametrize("tile_size", [2, 3, 4])
+@pytest.mark.parametrize("tile_size", [2, 3, 4, 6, 8])
 def test_tiled_launch_plans_agree(synth_model, tile_size, plan):
     forest = model_io.load_xgboost_json(synth_model(2))
     x = synth.CONFIGS[2].batch_rows(1501, seed_offset=6)
@@ -900,14 +952,16 @@ def test_tiled_launch_plans_agree(synth_model, tile_size, plan):
     x[4, :] = -np.inf
     x[5, :] = np.nan
     runner = make_tiled_runner(synth_model(2), 1501, tile_size)
+    if tile_size > 4 and plan[3] < 24576:        # the biggest tree of this model takes 18 KB in 64-byte tiles
+        plan = (128, 2, 1, 32768, 1)
     runner.set_plan(*plan)
     assert " tileSize=%d " % tile_size in runner.describe_plan()
     check_against_oracle(runner, forest, x)
 
 
 def test_tile_sizes_the_kernels_do_not_walk_are_refused(synth_model):
-    with pytest.raises(RuntimeError, match="tile size 8 is not supported"):
-        make_tiled_runner(synth_model(1), 64, 8)
+    with pytest.raises(RuntimeError, match="tile size 9 is not supported"):
+        make_tiled_runner(synth_model(1), 64, 9)         # the reference's own look-up table stops at 8 (256 outcomes per shape)
     with pytest.raises(RuntimeError, match="row tile below 64 KB"):
         make_tiled_runner(synth_model(4), 64, 2)          # 2000 features: no tiled row tile
     runner = make_tiled_runner(synth_model(1), 64, 2)
@@ -941,6 +995,27 @@ def test_profiled_runner_selects_the_same_leaves(synth_model, plain_file, tmp_pa
     runner = make_tiled_runner(higgs, hx.shape[0], tile_size, tiling_type, higgs_profile, peel)
     np.testing.assert_array_equal(gpu_leaf_ids(runner, hx), cpu_oracle.leaf_ids(hforest, hx))
     np.testing.assert_allclose(gpu_predict(runner, hx), data[:, -1], rtol=RTOL_SUM, atol=ATOL_PROB)
+
+
+def test_describe_plan_says_where_walk_peeling_applies(synth_model, tmp_path):
+    """Peeled walks exist for the tiled kernel and for the scalar row-parallel kernel that stores sums; a
+    classifier whose walk kernel keeps the arg-max itself walks every bundle to its full depth, and says so."""
+    forest = model_io.load_xgboost_json(synth_model(3))
+    x = synth.CONFIGS[3].batch_rows(1000, seed_offset=3)
+    profile = write_profile(tmp_path / "c3.profile.csv", forest, cpu_oracle.leaf_ids(forest, synth.CONFIGS[3].batch_rows(2000)))
+    runner = make_tiled_runner(synth_model(3), 1000, 1, 1, profile, True, multiclass=True)
+    assert " peelWalks=ignored(fused) " in runner.describe_plan()
+    check_against_oracle(runner, forest, x)
+    runner.set_plan(128, 8, 4, 0, 2)                  # two tree slices: sums go through the finalize kernel
+    assert " peelWalks=1 " in runner.describe_plan()
+    check_against_oracle(runner, forest, x)
+    runner.set_tree_parallel_plan(4, 64, 1, 0, 1)
+    assert " peelWalks=ignored(tree_parallel) " in runner.describe_plan()
+    tiled = make_tiled_runner(synth_model(3), 1000, 4, 1, profile, True, multiclass=True)
+    assert " peelWalks=1 " in tiled.describe_plan()
+    check_against_oracle(tiled, forest, x)
+    with pytest.raises(RuntimeError, match="row-parallel"):
+        tiled.set_global_walk_plan(256, 4, 1)         # a tiled runner does not quietly become a scalar walk
 
 
 @pytest.mark.parametrize("features,rows", [(20000, 300), (40000, 70)])

@@ -117,6 +117,100 @@ def test_onnx_comparison_modes_and_encodings(lib, tmp_path, mode, packed):
     lib.tbmi_delete_forest(h)
 
 
+def preorder_trees(rng, count, num_features, max_depth=5):
+    """Random trees numbered in pre-order (node, left subtree, right subtree) - the numbering both ONNX loaders
+    give their nodes (src/json/onnxmodelparser.h:315-334) - so that a loaded tree can be compared with what
+    the writer was handed index by index."""
+    trees = []
+    for _ in range(count):
+        value, feature, left, right = [], [], [], []
+
+        def grow(depth):
+            me = len(value)
+            value.append(0.0); feature.append(0); left.append(-1); right.append(-1)
+            if depth < max_depth and (depth == 0 or rng.random() < 0.7):
+                value[me] = float(np.float32(rng.normal()))
+                feature[me] = int(rng.integers(0, num_features))
+                left[me] = grow(depth + 1)
+                right[me] = grow(depth + 1)
+            else:
+                value[me] = float(np.float32(rng.normal(0.0, 0.3)))
+            return me
+
+        grow(0)
+        trees.append((np.asarray(value, np.float32), np.asarray(feature, np.int32), left, right))
+    return trees
+
+
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("post_transform,transform", [("NONE", model_io.IDENTITY), ("LOGISTIC", model_io.SIGMOID),
+                                                      ("SOFTMAX", model_io.SOFTMAX)])
+def test_onnx_classifier_comes_back_as_written(lib, tmp_path, post_transform, transform, packed):
+    """TreeEnsembleClassifier (src/json/onnxmodelparser.h:102-113 post_transform, :162-172 n_targets only counts
+    for classifiers, :355-374 one class id per tree): the forest handed to the writer - thresholds, features,
+    links, leaf weights, class id per tree, base value, transform - comes back field for field from the C++
+    loader and from the oracle's loader, and the oracle's class ids on that forest are those of the reference's
+    own DecisionForest::Predict_Float fed the same arrays through NewTree/NewNode."""
+    from oracle import cpu_oracle
+    rng = np.random.Generator(np.random.PCG64(31 + len(post_transform)))
+    classes, features = 5, 6
+    trees = preorder_trees(rng, 23, features)
+    class_ids = [int(c) for c in rng.integers(0, classes, len(trees))]
+    path = tmp_path / "classifier.onnx"
+    write_onnx(path, trees, base_value=0.125, post_transform=post_transform, classifier=True, n_classes=classes,
+               class_ids=class_ids, packed=packed)
+    written = model_io._assemble([(t[0].astype(np.float64), t[1], t[2], t[3]) for t in trees], num_features=features,
+                                 initial_value=0.125, transform=transform, num_classes=classes, predicate=model_io.PRED_LT,
+                                 class_id=np.asarray(class_ids, np.int32), meta={})
+    loaded = model_io.load_onnx(path, features)
+    assert (loaded.num_trees, loaded.num_features, loaded.num_classes, loaded.transform, loaded.predicate,
+            loaded.initial_value) == (len(trees), features, classes, transform, model_io.PRED_LT, 0.125)
+    np.testing.assert_array_equal(loaded.class_id, class_ids)
+    for t in range(len(trees)):
+        for got, want in zip(loaded.tree(t), written.tree(t)):          # thresholds / leaf weights, features, left, right
+            np.testing.assert_array_equal(got, want)
+    h = load_forest(lib, path, "onnx_file", features)
+    assert_same_forest(lib, h, written)
+    lib.tbmi_delete_forest(h)
+    # a regressor with the same attributes has no classes (n_targets is looked at for classifiers only)
+    write_onnx(tmp_path / "regressor.onnx", trees, base_value=0.125, post_transform="NONE", classifier=False, n_classes=classes,
+               class_ids=class_ids, packed=packed)
+    assert model_io.load_onnx(tmp_path / "regressor.onnx", features).num_classes == 0
+    h = load_forest(lib, tmp_path / "regressor.onnx", "onnx_file", features)
+    info, _, _ = forest_arrays(lib, h)
+    assert info[2] == 0
+    lib.tbmi_delete_forest(h)
+    # class ids of the oracle on the loaded forest = the reference's own walk + per-class sums + arg-max
+    x = rng.normal(size=(500, features)).astype(np.float32)
+    pred, sums = cpu_oracle.predict(loaded, x)
+    top2 = np.sort(sums, axis=1)[:, -2:]
+    assert (top2[:, 1] > top2[:, 0]).all()            # no exact ties: the two tie rules do not come into play
+    np.testing.assert_array_equal(pred, np.argmax(sums, axis=1))
+    if cpu_oracle.ref_available():
+        as_softmax = model_io._assemble([(t[0].astype(np.float64), t[1], t[2], t[3]) for t in trees], num_features=features,
+                                        initial_value=0.125, transform=model_io.SOFTMAX, num_classes=classes,
+                                        predicate=model_io.PRED_LT, class_id=np.asarray(class_ids, np.int32), meta={})
+        ref = cpu_oracle.RefForest(as_softmax)        # (Predict_Float insists on the soft-max transform for classifiers)
+        np.testing.assert_array_equal(ref.predict_float(x), pred.astype(np.float32))
+        np.testing.assert_array_equal(ref.predict_double(x.astype(np.float64)), pred.astype(np.float64))
+
+
+def test_onnx_classifier_with_several_class_ids_in_one_tree_is_refused(lib, tmp_path):
+    """src/json/onnxmodelparser.h:364-367 asserts one class id per tree; here the loaders say so."""
+    rng = np.random.Generator(np.random.PCG64(5))
+    trees = preorder_trees(rng, 4, 3)
+    path = tmp_path / "mixed.onnx"
+    write_onnx(path, trees, classifier=True, n_classes=3, class_ids=[0, 1, [0, 2], 1])
+    assert lib.tbmi_load_forest(str(path).encode(), b"onnx_file", 3) == 0
+    assert "multiple class IDs per tree" in last_error()
+    with pytest.raises(AssertionError):
+        model_io.load_onnx(path, 3)
+    write_onnx(path, trees, classifier=False, n_classes=3, class_ids=[0, 1, [0, 2], 1])       # regressors do not look
+    assert model_io.load_onnx(path, 3).num_classes == 0
+    h = load_forest(lib, path, "onnx_file", 3)
+    lib.tbmi_delete_forest(h)
+
+
 def test_global_layout_round_trips(lib, synth_model):
     for k in (1, 3, 5):
         h = load_forest(lib, synth_model(k))

@@ -1,6 +1,7 @@
 """The entry point that allocates nothing (tbmi_run_device_noalloc) against tbmi_run_device, through the C ABI:
 bit-equal results on two calls in a row, the second with a smaller input, for plans whose kernels use scratch
-memory (classifier partial sums, tree slices, rank-quantised rows) and for one that uses none."""
+memory (classifier partial sums, tree slices, rank-quantised rows) and for one that uses none - and both
+against the CPU oracle on the same rows."""
 import numpy as np
 import pytest
 
@@ -8,6 +9,7 @@ pytestmark = pytest.mark.gpu
 
 torch = pytest.importorskip("torch")
 
+from oracle import cpu_oracle, model_io  # noqa: E402
 from treebeard_amd import synth, treebeard  # noqa: E402
 from treebeard_amd.runtime_api import api  # noqa: E402
 
@@ -52,10 +54,18 @@ def test_no_alloc_entry_point_matches_run_device(synth_model, k, plan, first, se
         runner.set_plan(*plan[1:])
     elif plan:
         runner.set_tree_parallel_plan(*plan[1:])
+    forest = model_io.load_xgboost_json(synth_model(k))
     for call, rows in enumerate((first, second)):
         x = synth.CONFIGS[k].batch_rows(rows, seed_offset=11 + call)
         got, want = _both(runner, x)
         np.testing.assert_array_equal(got, want)
+        pred, _ = cpu_oracle.predict(forest, x)         # the oracle itself, not only the allocating entry point
+        if forest.num_classes > 0:
+            np.testing.assert_array_equal(got.astype(np.float32), pred)
+        elif forest.transform == model_io.SIGMOID:
+            np.testing.assert_allclose(got, pred, rtol=0, atol=1e-6)
+        else:
+            np.testing.assert_allclose(got, pred, rtol=1e-5, atol=0)
 
 
 def test_no_alloc_entry_point_rejects_what_does_not_fit(synth_model):

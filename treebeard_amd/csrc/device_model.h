@@ -23,7 +23,7 @@
 //    dependency chains.  A bundle records the K root addresses, the trip count
 //    (deepest tree of the bundle) and the class the trees add to.
 //
-// Tiled layout (LaunchPlan::tileSize T in {2, 3, 4}; the reference's tile of T connected internal nodes,
+// Tiled layout (LaunchPlan::tileSize T in 2..8; the reference's tile of T connected internal nodes,
 // src/mlir/UniformTilingTransformation.cpp:148-195, src/mlir/ProbabilityBasedTilingTransform.cpp:124-198):
 //  * A TILE holds its nodes in level order, struct-of-arrays: T thresholds, T feature offsets, the byte
 //    address of its first child tile and a child-select table, in 16 / 24 / 32 bytes for T = 2 / 3 / 4:
@@ -40,6 +40,17 @@
 //  * Unused node slots of a short tile test the pad feature; their outcome bits are don't-cares of `select`.
 //  * A leaf is a tile of its own: thr[0] is the prediction, every slot tests the pad feature, childBase is
 //    the tile's own address and select is 0, so a walk of `depth` tile steps needs no leaf test either.
+//  * Tile sizes 5 to 8 share one 64-byte tile of eight slots (four 16-byte reads), the reference's default
+//    tile size 8 among them (test/python/cpu_tests.py:14, src/test/GPUTests.cpp:995):
+//      { f32 thr[8]; u16 off[8]; u64 links; u16 childBase; u16 pad[3] }
+//    A table of 256 outcomes does not fit a tile, and one row of the reference's LUT per shape present in a
+//    model (1430 shapes of 256 entries) fits no LDS, so the tile carries its own shape instead: `links` holds
+//    two 4-bit links per slot, nibble 2 s + 1 taken when slot s sends the row left (its outcome bit is set) and
+//    nibble 2 s when it sends it right.  A link below 7 names the next slot (link + 1: slot 0 is nobody's
+//    child), a link of 7 or more the child reached (link - 7, children numbered left to right, 0..8).  The
+//    walk follows at most eight links from slot 0; this is the reference's LUT[shape][outcome] evaluated
+//    instead of stored, so the outcome bit order and the child numbering are the same.  A leaf tile's links
+//    all say "child 0" and its childBase is its own address.
 #pragma once
 
 #include <cstdint>
@@ -48,11 +59,18 @@ namespace tbamd {
 
 constexpr int kMaxInterleave = 8;
 constexpr uint32_t kNodeBytes = 8;
-constexpr int kMaxTileSize = 4;
+constexpr int kMaxTileSize = 8;
+// Tiles of more than kMaxSelectTile nodes carry links instead of a child-select table.
+constexpr int kMaxSelectTile = 4;
 // Bytes of one tile of T nodes (T = 1 is the scalar node).
-constexpr uint32_t TileBytes(int tileSize) { return tileSize <= 1 ? kNodeBytes : tileSize == 2 ? 16u : tileSize == 3 ? 24u : 32u; }
-// Width of one field of a tile's child-select table.
+constexpr uint32_t TileBytes(int tileSize) {
+  return tileSize <= 1 ? kNodeBytes : tileSize == 2 ? 16u : tileSize == 3 ? 24u : tileSize == 4 ? 32u : 64u;
+}
+// Width of one field of a tile's child-select table (tiles of up to kMaxSelectTile nodes).
 constexpr uint32_t TileSelectBits(int tileSize) { return tileSize == 4 ? 3u : 2u; }
+// Links of the 64-byte tile: values below kTileLinkExit name a slot (value + 1), the others a child (value - kTileLinkExit).
+constexpr uint32_t kTileLinkExit = 7;
+constexpr uint64_t kLeafTileLinks = 0x7777777777777777ull; // every link: child 0
 
 struct DeviceNode {
   float value;

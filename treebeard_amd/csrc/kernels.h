@@ -69,8 +69,8 @@ struct FinalizeParams {
 // `interleave` in {1,2,4,8}; `tileMode`: 0 f32 tile with byte offsets, 1 f32 tile with offsets in units of
 // 4 bytes, 2 one-byte rank tile (p.x then points at the output of LaunchBinRows; 64 rows per block).
 hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, int tileMode, size_t ldsBytes, hipStream_t stream);
-// The same block shape over tiled trees (tiles of 2, 3 or 4 nodes, f32 row tile with byte offsets below 64 KB);
-// `interleave` in {1,2,4}.
+// The same block shape over tiled trees (tiles of 2 to 8 nodes, f32 row tile with byte offsets below 64 KB);
+// `interleave` in {1,2,4}.  Tree groups are staged by direct global-to-LDS copies.
 hipError_t LaunchWalkRowsTiled(const WalkParams &p, int tileSize, int interleave, size_t ldsBytes, hipStream_t stream);
 // Rank-quantises rows x[rows][numFeatures] into ranks[ceil(rows/64)][numFeatures][64] (bytes) with the
 // packer's threshold table ([chunk][k][64], +inf padded, tableDepth = 2^n - 1).

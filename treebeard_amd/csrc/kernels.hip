@@ -379,14 +379,15 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
 }
 
 // ---------------------------------------------------------------------------
-// Row-parallel walk over TILED trees (tiles of T = 2, 3 or 4 nodes, layout in device_model.h): the
+// Row-parallel walk over TILED trees (tiles of T = 2 to 8 nodes, layout in device_model.h): the
 // reference's tile step (src/mlir/CodeGenStateMachine.cpp:284-506, cooperative GPU form
 // src/gpu/GPUSimtPass.cpp:39-133) as branch-free per-lane code.  One step reads the tile (thresholds,
-// feature offsets, child base and the tile's own child-select row) with one or two wide LDS reads, gathers
+// feature offsets, child base and the tile's own child-select row) with one to four wide LDS reads, gathers
 // the T feature values of the lane's row, turns the T comparisons into an outcome word (node i in bit i)
-// and picks the child out of the select row with one shift.  Leaves are tiles that select themselves, so a
-// bundle walks `depth` tile steps without a leaf test.  Block shape, row tile, tree groups, tree threads,
-// class flush and epilogue are those of WalkRowsLdsKernel.
+// and picks the child out of the select row with one shift (tiles of up to 4 nodes) or by following the
+// tile's links (the eight-slot tile of tile sizes 5 to 8).  Leaves are tiles that select themselves, so a
+// bundle walks `depth` tile steps without a leaf test.  Block shape, row tile, tree groups (staged by direct
+// global-to-LDS copies), tree threads, class flush and epilogue are those of WalkRowsLdsKernel.
 //
 // Bundles carry a peel depth (taken from a hit-count profile: the steps that bring 90 % of the profiled
 // rows to a leaf, src/mlir/ProbabilityBasedTilingTransform.cpp:66-73; equal to the depth without one): the
@@ -396,30 +397,39 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
 typedef const __attribute__((address_space(3))) U32x4 *LdsQuadPtr;
 __device__ __forceinline__ U32x4 LdsLoadQuad(uint32_t address) { return *(LdsQuadPtr)(uintptr_t)address; }
 
-template <int T>
+template <int T> // 2, 3, 4, or kMaxTileSize for the eight-slot tile of tile sizes 5 to 8
 __device__ __forceinline__ uint32_t TileStep(uint32_t addr, uint32_t column) {
+  static_assert(T >= 2 && (T <= kMaxSelectTile || T == kMaxTileSize), "tile sizes 5 to 8 share the eight-slot tile");
   float thr[T];
   uint32_t off[T];
   uint32_t childBase;
-  uint64_t select;
-  if (T == 2) {
+  uint64_t select; // the child-select row, or the links of the eight-slot tile
+  if constexpr (T == 2) {
     const U32x4 q = LdsLoadQuad(addr);
     thr[0] = AsFloat(q.x), thr[1] = AsFloat(q.y);
     off[0] = q.z & 0xFFFFu, off[1] = q.z >> 16;
     childBase = q.w & 0xFFFFu;
     select = q.w >> 16;
-  } else if (T == 3) {
+  } else if constexpr (T == 3) {
     const U32x2 a = LdsLoadNode(addr), b = LdsLoadNode(addr + 8), c = LdsLoadNode(addr + 16);
     thr[0] = AsFloat(a.x), thr[1] = AsFloat(a.y), thr[2] = AsFloat(b.x);
     off[0] = b.y & 0xFFFFu, off[1] = b.y >> 16, off[2] = c.x & 0xFFFFu;
     childBase = c.x >> 16;
     select = c.y & 0xFFFFu;
-  } else {
+  } else if constexpr (T == 4) {
     const U32x4 q0 = LdsLoadQuad(addr), q1 = LdsLoadQuad(addr + 16);
     thr[0] = AsFloat(q0.x), thr[1] = AsFloat(q0.y), thr[2] = AsFloat(q0.z), thr[3] = AsFloat(q0.w);
     off[0] = q1.x & 0xFFFFu, off[1] = q1.x >> 16, off[2] = q1.y & 0xFFFFu, off[3] = q1.y >> 16;
     childBase = q1.z & 0xFFFFu;
     select = (uint64_t)(q1.z >> 16) | ((uint64_t)q1.w << 16);
+  } else {
+    const U32x4 q0 = LdsLoadQuad(addr), q1 = LdsLoadQuad(addr + 16), q2 = LdsLoadQuad(addr + 32), q3 = LdsLoadQuad(addr + 48);
+    thr[0] = AsFloat(q0.x), thr[1] = AsFloat(q0.y), thr[2] = AsFloat(q0.z), thr[3] = AsFloat(q0.w);
+    thr[4] = AsFloat(q1.x), thr[5] = AsFloat(q1.y), thr[6] = AsFloat(q1.z), thr[7] = AsFloat(q1.w);
+    off[0] = q2.x & 0xFFFFu, off[1] = q2.x >> 16, off[2] = q2.y & 0xFFFFu, off[3] = q2.y >> 16;
+    off[4] = q2.z & 0xFFFFu, off[5] = q2.z >> 16, off[6] = q2.w & 0xFFFFu, off[7] = q2.w >> 16;
+    select = (uint64_t)q3.x | ((uint64_t)q3.y << 32);
+    childBase = q3.z & 0xFFFFu;
   }
   uint32_t outcome = 0;
 #pragma unroll
@@ -427,11 +437,24 @@ __device__ __forceinline__ uint32_t TileStep(uint32_t addr, uint32_t column) {
     const float x = LdsLoadFloat(column + off[i]);
     outcome |= (x < thr[i] ? 1u : 0u) << i;
   }
-  const uint32_t child = (uint32_t)(select >> (outcome * TileSelectBits(T))) & ((1u << TileSelectBits(T)) - 1u);
-  return childBase + child * TileBytes(T);
+  if constexpr (T > kMaxSelectTile) {
+    // Follow the tile's links from slot 0: nibble 2 s + 1 when slot s sends the row left, nibble 2 s otherwise; a
+    // link below kTileLinkExit names the next slot, the others the child.  Eight slots: at most eight links.
+    uint32_t link = (uint32_t)(select >> ((outcome & 1u) << 2)) & 15u;
+#pragma unroll
+    for (int hop = 1; hop < T; ++hop) {
+      const uint32_t slot = (link + 1u) & 7u;
+      const uint32_t next = (uint32_t)(select >> (slot * 8u + (((outcome >> slot) & 1u) << 2))) & 15u;
+      link = link < kTileLinkExit ? next : link;
+    }
+    return childBase + (link - kTileLinkExit) * TileBytes(T);
+  } else {
+    const uint32_t child = (uint32_t)(select >> (outcome * TileSelectBits(T))) & ((1u << TileSelectBits(T)) - 1u);
+    return childBase + child * TileBytes(T);
+  }
 }
 
-template <int T, int K, int PF, int kVariant> // kVariant: kWalkPlain, kWalkDump or kWalkFuse (the peel tail is always there)
+template <int T, int K, int kVariant> // kVariant: kWalkPlain, kWalkDump or kWalkFuse (the peel tail is always there)
 __global__ void __launch_bounds__(1024)
 WalkRowsTiledKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16,
                     const DeviceBundle *__restrict__ bundles, const DeviceGroup *__restrict__ groups,
@@ -468,17 +491,6 @@ WalkRowsTiledKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes
   int curClass = 0;
   float best = -INFINITY; // fuseArgmax: running maximum of the class sums and its class (tree thread 0)
   int bestClass = 0;
-  U32x4 fetched[PF];
-#define TBAMD_PREFETCH_GROUP(NEXTGRP)                                                                                  \
-  {                                                                                                                    \
-    const DeviceGroup nextGrp = (NEXTGRP);                                                                             \
-    const U32x4 *src = reinterpret_cast<const U32x4 *>(nodes16) + (nextGrp.nodeBegin >> 1);                            \
-    const int last = (int)(nextGrp.nodeCount >> 1) - 1;                                                                \
-    _Pragma("unroll") for (int i = 0; i < PF; ++i) {                                                                   \
-      const int idx = tid + i * threads;                                                                               \
-      fetched[i] = src[idx < last ? idx : last];                                                                       \
-    }                                                                                                                  \
-  }
 #define TBAMD_FLUSH_CLASS(UPTO)                                                                                        \
   {                                                                                                                    \
     if (TT > 1) {                                                                                                      \
@@ -504,22 +516,22 @@ WalkRowsTiledKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes
     }                                                                                                                  \
     acc = 0.0;                                                                                                         \
   }
-  if (gBegin < gEnd) TBAMD_PREFETCH_GROUP(groups[gBegin])
-
   for (int g = gBegin; g < gEnd; ++g) {
     const DeviceGroup grp = groups[g];
     __syncthreads();
     {
-      U32x4 *dst = reinterpret_cast<U32x4 *>(lds);
+      // The group goes straight from global memory into LDS (lane i of a wave-wide load leaves its 16 bytes at
+      // base + 16 i, lanes switched off write nothing), as in the scalar kernel's direct form.
+      const U32x4 *src = reinterpret_cast<const U32x4 *>(nodes16) + (grp.nodeBegin >> 1);
       const int pieces = (int)(grp.nodeCount >> 1);
-#pragma unroll
-      for (int i = 0; i < PF; ++i) {
-        const int idx = tid + i * threads;
-        if (idx < pieces) dst[idx] = fetched[i];
-      }
+      const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+      for (int first = wave * 64; first < pieces; first += threads)
+        if (first + (tid & 63) < pieces)
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + first + (tid & 63)),
+                                           (__attribute__((address_space(3))) void *)(lds + (uint32_t)first * 16u), 16, 0, 0);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     __syncthreads();
-    if (g + 1 < gEnd) TBAMD_PREFETCH_GROUP(groups[g + 1])
 
     uint32_t b0 = 0;
     while (b0 < grp.bundleCount) {
@@ -596,7 +608,6 @@ WalkRowsTiledKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes
     out[row] = (float)(s.transform == 1 ? 1.0 / (1.0 + exp(-margin)) : margin);
   }
 #undef TBAMD_FLUSH_CLASS
-#undef TBAMD_PREFETCH_GROUP
 }
 
 // ---------------------------------------------------------------------------
@@ -1119,40 +1130,31 @@ hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, int tileMode, 
 }
 
 namespace {
-template <int T, int K, int PF, int V>
+template <int T, int K, int V>
 hipError_t LaunchTiledVariant(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
-  hipError_t e = AllowFullLds<&WalkRowsTiledKernel<T, K, PF, V>>();
+  hipError_t e = AllowFullLds<&WalkRowsTiledKernel<T, K, V>>();
   if (e != hipSuccess) return e;
-  WalkRowsTiledKernel<T, K, PF, V><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out, p.classOut, p.partial,
-                                                                      p.leafIds, p.nodeOrigin, p.slotTree);
+  WalkRowsTiledKernel<T, K, V><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.groups, p.s, p.out, p.classOut, p.partial,
+                                                                  p.leafIds, p.nodeOrigin, p.slotTree);
   return hipGetLastError();
 }
 
-template <int T, int K, int PF>
-hipError_t LaunchTiledTKP(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
+template <int T, int K>
+hipError_t LaunchTiledTK(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
   if (p.leafIds) {
     if (p.s.fuseArgmax) return hipErrorInvalidValue;
-    return LaunchTiledVariant<T, K, PF, kWalkDump>(p, grid, block, ldsBytes, stream);
+    return LaunchTiledVariant<T, K, kWalkDump>(p, grid, block, ldsBytes, stream);
   }
-  if (p.s.fuseArgmax) return LaunchTiledVariant<T, K, PF, kWalkFuse>(p, grid, block, ldsBytes, stream);
-  return LaunchTiledVariant<T, K, PF, kWalkPlain>(p, grid, block, ldsBytes, stream);
-}
-
-template <int T, int K>
-hipError_t LaunchTiledTK(const WalkParams &p, int prefetch, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
-  if (prefetch <= 4) return LaunchTiledTKP<T, K, 4>(p, grid, block, ldsBytes, stream);
-  if (prefetch <= 8) return LaunchTiledTKP<T, K, 8>(p, grid, block, ldsBytes, stream);
-  if (prefetch <= 16) return LaunchTiledTKP<T, K, 16>(p, grid, block, ldsBytes, stream);
-  return hipErrorInvalidValue;
+  if (p.s.fuseArgmax) return LaunchTiledVariant<T, K, kWalkFuse>(p, grid, block, ldsBytes, stream);
+  return LaunchTiledVariant<T, K, kWalkPlain>(p, grid, block, ldsBytes, stream);
 }
 
 template <int T>
-hipError_t LaunchTiledT(const WalkParams &p, int interleave, int prefetch, dim3 grid, dim3 block, size_t ldsBytes,
-                        hipStream_t stream) {
+hipError_t LaunchTiledT(const WalkParams &p, int interleave, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
   switch (interleave) {
-  case 1: return LaunchTiledTK<T, 1>(p, prefetch, grid, block, ldsBytes, stream);
-  case 2: return LaunchTiledTK<T, 2>(p, prefetch, grid, block, ldsBytes, stream);
-  case 4: return LaunchTiledTK<T, 4>(p, prefetch, grid, block, ldsBytes, stream);
+  case 1: return LaunchTiledTK<T, 1>(p, grid, block, ldsBytes, stream);
+  case 2: return LaunchTiledTK<T, 2>(p, grid, block, ldsBytes, stream);
+  case 4: return LaunchTiledTK<T, 4>(p, grid, block, ldsBytes, stream);
   default: return hipErrorInvalidValue;
   }
 }
@@ -1167,12 +1169,13 @@ hipError_t LaunchWalkRowsTiled(const WalkParams &p, int tileSize, int interleave
   if ((int64_t)(p.s.numFeatures + 1) * RB * 4 > 0x10000) return hipErrorInvalidValue;
   const int64_t blocks = (p.s.rows + RB - 1) / RB;
   if (blocks > 0x7FFFFFFF || p.s.treeSlices < 1 || p.s.treeSlices > 65535) return hipErrorInvalidValue;
-  const int prefetch = (int)((p.s.groupRegionBytes / 16 + RB * TT - 1) / (RB * TT));
   dim3 grid((unsigned)blocks, (unsigned)p.s.treeSlices), block((unsigned)(RB * TT));
   switch (tileSize) {
-  case 2: return LaunchTiledT<2>(p, interleave, prefetch, grid, block, ldsBytes, stream);
-  case 3: return LaunchTiledT<3>(p, interleave, prefetch, grid, block, ldsBytes, stream);
-  case 4: return LaunchTiledT<4>(p, interleave, prefetch, grid, block, ldsBytes, stream);
+  case 2: return LaunchTiledT<2>(p, interleave, grid, block, ldsBytes, stream);
+  case 3: return LaunchTiledT<3>(p, interleave, grid, block, ldsBytes, stream);
+  case 4: return LaunchTiledT<4>(p, interleave, grid, block, ldsBytes, stream);
+  case 5: case 6: case 7: case 8: // one eight-slot tile for all four; the packer fills as many slots as the tile size says
+    return LaunchTiledT<kMaxTileSize>(p, interleave, grid, block, ldsBytes, stream);
   default: return hipErrorInvalidValue;
   }
 }

@@ -106,7 +106,8 @@ struct TileInfo {
   int32_t exits[kMaxTileSize + 1] = {};    // original node ids the tile's children start at, left to right
   int32_t leafNode = -1;                   // leaf tiles: the original leaf
   uint32_t firstChild = 0;                 // tile index (inside the tree) of child 0; own index on a leaf tile
-  uint64_t select = 0;                     // child number per outcome word, TileSelectBits() each
+  uint64_t select = 0;                     // child number per outcome word, TileSelectBits() each (tiles of up to 4 nodes)
+  uint64_t links = kLeafTileLinks;         // two 4-bit links per slot (tiles of 5 to 8 nodes, device_model.h)
   int32_t depth = 0;                       // tile steps from this tile down to its deepest leaf
   int32_t level = 0;                       // tile steps from the root tile
 };
@@ -262,17 +263,27 @@ TiledTree TileTree(const Tree &tree, int T, int tiling, const std::vector<int64_
         }
       }
     }
-    // the tile's row of the child look-up table: outcome bit i set = node i sends the row left
-    const uint32_t width = TileSelectBits(T);
-    for (uint32_t outcome = 0; outcome < (1u << T); ++outcome) {
-      int slot = 0;
-      for (;;) {
-        const int32_t next = ((outcome >> slot) & 1u) ? leftSlot[slot] : rightSlot[slot];
-        if (next < 0) {
-          tile.select |= (uint64_t)(-next - 1) << (outcome * width);
-          break;
+    if (T <= kMaxSelectTile) {
+      // the tile's row of the child look-up table: outcome bit i set = node i sends the row left
+      const uint32_t width = TileSelectBits(T);
+      for (uint32_t outcome = 0; outcome < (1u << T); ++outcome) {
+        int slot = 0;
+        for (;;) {
+          const int32_t next = ((outcome >> slot) & 1u) ? leftSlot[slot] : rightSlot[slot];
+          if (next < 0) {
+            tile.select |= (uint64_t)(-next - 1) << (outcome * width);
+            break;
+          }
+          slot = next;
         }
-        slot = next;
+      }
+    } else {
+      // the tile's shape itself: per slot where a row goes when the slot's predicate holds (left) and when not
+      auto link = [](int32_t next) -> uint64_t { return next < 0 ? kTileLinkExit + (uint64_t)(-next - 1) : (uint64_t)(next - 1); };
+      tile.links = 0;
+      for (int slot = 0; slot < kMaxTileSize; ++slot) {
+        const uint64_t left = slot < n ? link(leftSlot[slot]) : kTileLinkExit, right = slot < n ? link(rightSlot[slot]) : kTileLinkExit;
+        tile.links |= (right << (8 * slot)) | (left << (8 * slot + 4));
       }
     }
     tile.firstChild = (uint32_t)roots.size();
@@ -297,7 +308,7 @@ void EmitTile(const Tree &tree, const TileInfo &tile, int T, uint32_t treeBase, 
   const uint32_t bytes = TileBytes(T);
   float thr[kMaxTileSize] = {};
   uint16_t off[kMaxTileSize];
-  for (int i = 0; i < T; ++i) off[i] = (uint16_t)padOffset;
+  for (int i = 0; i < kMaxTileSize; ++i) off[i] = (uint16_t)padOffset;
   if (tile.count == 0) {
     thr[0] = tree.value[tile.leafNode];
   } else {
@@ -310,6 +321,13 @@ void EmitTile(const Tree &tree, const TileInfo &tile, int T, uint32_t treeBase, 
   if (childAddress + (uint32_t)std::max(tile.numExits, 1) * bytes > 0x10000u) throw Error("internal error: tile address beyond the group");
   const uint16_t childBase = (uint16_t)childAddress;
   std::memset(dst, 0, bytes);
+  if (T > kMaxSelectTile) { // eight slots whatever the tile size: { thr[8]; off[8]; links; childBase }
+    std::memcpy(dst, thr, 32);
+    std::memcpy(dst + 32, off, 16);
+    std::memcpy(dst + 48, &tile.links, 8);
+    std::memcpy(dst + 56, &childBase, 2);
+    return;
+  }
   std::memcpy(dst, thr, (size_t)T * 4);
   std::memcpy(dst + T * 4, off, (size_t)T * 2);
   std::memcpy(dst + T * 6, &childBase, 2);
@@ -339,6 +357,13 @@ int32_t PeelDepth(const std::vector<int64_t> &hits, const std::vector<int32_t> &
 }
 
 } // namespace
+
+int64_t BiggestTiledTreeBytes(const Forest &forest, int tileSize) {
+  if (tileSize < 2 || tileSize > kMaxTileSize) throw Error("internal error: tile size out of range");
+  size_t most = 0;
+  for (const Tree &tree : forest.trees) most = std::max(most, TileTree(tree, tileSize, 0, nullptr).tiles.size());
+  return (int64_t)most * TileBytes(tileSize);
+}
 
 namespace {
 

@@ -33,7 +33,7 @@ struct LaunchPlan {
   // by the number of that feature's split thresholds that are <= it (one byte), which preserves the
   // outcome of every comparison; 64 rows of 1 byte per feature then fit LDS where 64 f32 rows do not.
   bool quantizedRows = false;
-  // Tiled walk (row-parallel kernel on f32 rows only): nodes per tile, 1 = scalar nodes.  How the members of a
+  // Tiled walk (row-parallel kernel on f32 rows only): nodes per tile (up to 8), 1 = scalar nodes.  How the members of a
   // tile are chosen follows the reference: 0 breadth first (src/mlir/UniformTilingTransformation.cpp:148-195),
   // 1 most-visited child first on trees whose profile is skewed, 2 the same but breadth first below nodes that
   // fewer than 20 % of the rows reach (src/mlir/ProbabilityBasedTilingTransform.cpp:124-198, :243-262); 1 and
@@ -104,6 +104,10 @@ struct PackedModel {
 
 // Largest number of distinct split thresholds any one feature has (after comparison normalisation).
 int32_t MaxThresholdsPerFeature(const Forest &forest);
+
+// Bytes of the biggest tree once tiled breadth first with `tileSize` (2..8) nodes per tile, leaf tiles included.
+// (Tiling by hit counts picks other members but much the same number of tiles.)
+int64_t BiggestTiledTreeBytes(const Forest &forest, int tileSize);
 
 // Throws tbamd::Error when the plan cannot hold the model (tree larger than a
 // group, feature offsets that do not fit 16 bits, ...).  `profile` (may be null) feeds the plan's

@@ -102,15 +102,34 @@ void InferenceRunner::InitDevice() {
   Check(hipGetDeviceProperties(&prop, 0), "hipGetDeviceProperties");
   m_limits.computeUnits = prop.multiProcessorCount;
   m_limits.ldsBytesPerBlock = (int32_t)std::min<size_t>(prop.sharedMemPerBlock, 160 * 1024);
-  (void)ScratchOfCurrentDevice(); // set-up: the no-allocation entry point finds its array's address ready
+  // Set-up: the no-allocation entry point finds its array's address ready.  A failure here is that entry
+  // point's business only (it looks the address up again and reports the error): other callers never need it.
+  try {
+    (void)ScratchOfCurrentDevice();
+  } catch (const Error &) {
+    (void)hipGetLastError();
+  }
   Check(hipStreamCreateWithFlags(&m_stream, hipStreamNonBlocking), "hipStreamCreate");
   Check(hipEventCreate(&m_evStart), "hipEventCreate");
   Check(hipEventCreate(&m_evStop), "hipEventCreate");
+  Check(hipEventCreateWithFlags(&m_asyncDone, hipEventDisableTiming), "hipEventCreate");
+}
+
+void InferenceRunner::OrderAfterAsyncCall(hipStream_t stream) {
+  if (!m_asyncPending || stream == m_asyncStream) return; // (calls on one stream are ordered by the stream)
+  Check(hipStreamWaitEvent(stream, m_asyncDone, 0), "hipStreamWaitEvent");
+}
+
+void InferenceRunner::WaitForAsyncCall() {
+  if (!m_asyncPending) return;
+  Check(hipEventSynchronize(m_asyncDone), "hipEventSynchronize");
+  m_asyncPending = false;
 }
 
 InferenceRunner::~InferenceRunner() { Release(); }
 
 void InferenceRunner::Release() noexcept {
+  if (m_asyncPending) (void)hipEventSynchronize(m_asyncDone); // kernels of an asynchronous call still read the model
   if (m_stream) (void)hipStreamSynchronize(m_stream);
   FreeModel();
   (void)hipFree(m_dPartial);
@@ -124,6 +143,7 @@ void InferenceRunner::Release() noexcept {
   if (m_copyStream) (void)hipStreamDestroy(m_copyStream);
   if (m_evStart) (void)hipEventDestroy(m_evStart);
   if (m_evStop) (void)hipEventDestroy(m_evStop);
+  if (m_asyncDone) (void)hipEventDestroy(m_asyncDone);
   if (m_stream) (void)hipStreamDestroy(m_stream);
 }
 
@@ -171,6 +191,7 @@ void InferenceRunner::Repack(const LaunchPlan &plan) {
   PackedModel next = PackForest(m_forest, plan, m_profile.get());
   // refuse before anything is freed: a plan that fails leaves the runner as it was
   if (next.LdsBytes() > (size_t)m_limits.ldsBytesPerBlock) throw Error("launch plan exceeds the LDS of one workgroup");
+  WaitForAsyncCall();
   Check(hipStreamSynchronize(m_stream), "hipStreamSynchronize");
   FreeModel();
   m_model = std::move(next);
@@ -193,6 +214,7 @@ size_t InferenceRunner::RanksBytes(int64_t rows) const {
 void InferenceRunner::EnsurePartial(int64_t rows) {
   const size_t need = PartialBytes(rows);
   if (need <= m_partialBytes) return;
+  WaitForAsyncCall();
   Check(hipStreamSynchronize(m_stream), "hipStreamSynchronize");
   (void)hipFree(m_dPartial);
   m_dPartial = nullptr;
@@ -204,6 +226,7 @@ void InferenceRunner::EnsurePartial(int64_t rows) {
 void InferenceRunner::EnsureRanks(int64_t rows) {
   const size_t need = RanksBytes(rows);
   if (need <= m_ranksBytes) return;
+  WaitForAsyncCall();
   Check(hipStreamSynchronize(m_stream), "hipStreamSynchronize");
   (void)hipFree(m_dRanks);
   m_dRanks = nullptr;
@@ -212,9 +235,11 @@ void InferenceRunner::EnsureRanks(int64_t rows) {
   m_ranksBytes = need;
 }
 
-InferenceRunner::Workspace InferenceRunner::OwnWorkspace(int64_t rows) {
+InferenceRunner::Workspace InferenceRunner::OwnWorkspace(int64_t rows, hipStream_t stream) {
   EnsurePartial(rows);
   EnsureRanks(rows);
+  // An asynchronous call on another stream may still use these buffers: `stream` waits for it on the device.
+  OrderAfterAsyncCall(stream);
   Workspace ws;
   ws.partial = m_dPartial;
   ws.ranks = m_dRanks;
@@ -249,7 +274,8 @@ void InferenceRunner::SetGroupStaging(int32_t mode) {
 
 bool InferenceRunner::DirectStaging() const {
   const LaunchPlan &plan = m_model.plan;
-  if (plan.kernel != LaunchPlan::Kernel::kRowParallelLds || plan.tileSize > 1) return false; // (only the scalar row-parallel walk has the form)
+  if (plan.kernel != LaunchPlan::Kernel::kRowParallelLds) return false; // (only the row-parallel walks have the form)
+  if (plan.tileSize > 1) return true;                                    // (the tiled walk has no other)
   if (m_groupStaging != 0) return m_groupStaging == 2;
   // Measured on MI355X (28 to 520 features, 600 to 1000 trees): 5 to 15 % faster with two blocks per CU,
   // 2 to 4 % slower with one, whose wait for the copy nothing covers.  (LDS is handed out in coarse pieces.)
@@ -328,7 +354,7 @@ void InferenceRunner::Launch(const float *deviceInputs, int64_t rows, float *out
 
 void InferenceRunner::RunDevice(const float *deviceInputs, void *deviceResults, int64_t rows) {
   const int runs = gMeasureGpuKernelTime ? std::max(1, gNumberOfKernelRuns) : 1;
-  const Workspace ws = OwnWorkspace(rows);
+  const Workspace ws = OwnWorkspace(rows, m_stream);
   if (gMeasureGpuKernelTime) Check(hipEventRecord(m_evStart, m_stream), "hipEventRecord");
   for (int i = 0; i < runs; ++i) {
     if (ClassIdsAsInt8())
@@ -348,13 +374,17 @@ void InferenceRunner::RunDevice(const float *deviceInputs, void *deviceResults, 
 void InferenceRunner::RunDeviceOnStream(const float *deviceInputs, void *deviceResults, int64_t rows, hipStream_t stream) {
   if (rows < 0) throw Error("negative row count");
   if (rows > 0 && (!deviceInputs || !deviceResults)) throw Error("null device buffer");
-  // Growing the runner's buffers waits for the runner's own stream only; an earlier call on another
-  // stream that still uses them must have finished before a call with more rows is made.
-  const Workspace ws = OwnWorkspace(rows);
+  if (rows == 0) return;
+  // The runner's own stream is idle here (every entry point that uses it waits for it before returning); an
+  // earlier asynchronous call may still be running on another stream and uses the same buffers.
+  const Workspace ws = OwnWorkspace(rows, stream);
   if (ClassIdsAsInt8())
     Launch(deviceInputs, rows, nullptr, static_cast<int8_t *>(deviceResults), nullptr, nullptr, nullptr, stream, ws);
   else
     Launch(deviceInputs, rows, static_cast<float *>(deviceResults), nullptr, nullptr, nullptr, nullptr, stream, ws);
+  Check(hipEventRecord(m_asyncDone, stream), "hipEventRecord");
+  m_asyncStream = stream;
+  m_asyncPending = true;
 }
 
 size_t InferenceRunner::NoAllocScratchBytes() { return kNoAllocScratchBytes; }
@@ -384,13 +414,13 @@ void InferenceRunner::RunDeviceNoAlloc(const float *deviceInputs, void *deviceRe
 void InferenceRunner::RunDeviceMulticlass(const float *deviceInputs, int64_t rows, int8_t *classIds, float *margins,
                                           float *probabilities) {
   if (m_forest.numClasses == 0) throw Error("model is not a multiclass classifier");
-  Launch(deviceInputs, rows, nullptr, classIds, margins, probabilities, nullptr, m_stream, OwnWorkspace(rows));
+  Launch(deviceInputs, rows, nullptr, classIds, margins, probabilities, nullptr, m_stream, OwnWorkspace(rows, m_stream));
   Check(hipStreamSynchronize(m_stream), "inference kernels");
 }
 
 void InferenceRunner::DumpLeafIds(const float *deviceInputs, int32_t *deviceLeafIds, int64_t rows) {
   // results of the prediction itself are discarded
-  const Workspace ws = OwnWorkspace(rows);
+  const Workspace ws = OwnWorkspace(rows, m_stream);
   float *scratch = nullptr;
   Check(hipMalloc(reinterpret_cast<void **>(&scratch), std::max<int64_t>(rows, 1) * sizeof(float)), "allocate scratch");
   try {
@@ -470,7 +500,7 @@ void InferenceRunner::RunHostChunk(const void *hostInputs, void *hostResults, in
       }
       if (!m_copier) m_copier.reset(new ParallelCopier((int)std::min(8u, std::max(1u, std::thread::hardware_concurrency()))));
     }
-    const Workspace ws = OwnWorkspace(perPiece); // the pieces run one after the other on the runner's stream
+    const Workspace ws = OwnWorkspace(perPiece, m_stream); // the pieces run one after the other on the runner's stream
     int p = 0;
     for (int64_t first = 0; first < rows; first += perPiece, ++p) {
       const int64_t count = std::min(perPiece, rows - first);
@@ -497,7 +527,7 @@ void InferenceRunner::RunHostChunk(const void *hostInputs, void *hostResults, in
 void InferenceRunner::TimeKernels(const float *deviceInputs, void *deviceResults, int64_t rows, int32_t runs,
                                   double *walkMs, double *finalizeMs, double *binMs) {
   runs = std::max(1, runs);
-  const Workspace ws = OwnWorkspace(rows);
+  const Workspace ws = OwnWorkspace(rows, m_stream);
   const bool fused = FusesArgmax();
   const bool finalize = NeedsFinalize() && !fused;
   float ms = 0.f;
@@ -580,6 +610,18 @@ double InferenceRunner::AutoTune(const float *deviceInputs, int64_t rows) {
 std::string InferenceRunner::DescribePlan() const {
   std::ostringstream os;
   const LaunchPlan &p = m_model.plan;
+  // Walk peeling as the launch will apply it: the tiled walk and the scalar row-parallel walk on an f32 tile
+  // with byte offsets have the peeled form; the other walks take every bundle to its full depth.
+  std::string peel = "0";
+  if (p.peelWalks) {
+    if (p.kernel == LaunchPlan::Kernel::kTreeParallel) peel = "ignored(tree_parallel)";
+    else if (p.kernel == LaunchPlan::Kernel::kGlobalWalk) peel = "ignored(global_walk)";
+    else if (p.tileSize > 1) peel = "1";
+    else if (FusesArgmax()) peel = "ignored(fused)";
+    else if (p.quantizedRows) peel = "ignored(ranks)";
+    else if (p.featureOffsetInWords) peel = "ignored(words)";
+    else peel = "1";
+  }
   os << "kernel="
      << (p.kernel == LaunchPlan::Kernel::kTreeParallel ? "tree_parallel"
          : p.kernel == LaunchPlan::Kernel::kGlobalWalk ? "global_walk"
@@ -592,7 +634,7 @@ std::string InferenceRunner::DescribePlan() const {
      << " bundles=" << m_model.bundles.size() << " nodes=" << m_model.nodes.size()
      << " ldsBytes=" << m_model.LdsBytes() << " tileSize=" << p.tileSize << " tiling=" << p.tiling
      << " staging=" << (DirectStaging() ? "direct" : "registers")
-     << " peelWalks=" << (p.peelWalks ? 1 : 0) << " treesTiledByProfile=" << m_model.treesTiledByProfile
+     << " peelWalks=" << peel << " treesTiledByProfile=" << m_model.treesTiledByProfile
      << " lockStepSteps=" << m_model.lockStepSteps << " profiledSteps=" << m_model.profiledSteps;
   return os.str();
 }

@@ -50,6 +50,9 @@ public:
   void RunDevice(const float *deviceInputs, void *deviceResults, int64_t rows);
   // The same kernels enqueued on the caller's stream; returns without waiting for them.  Work the caller
   // queued on that stream before the call is seen by the kernels, work queued after it sees their results.
+  // The runner's buffers (model, partial sums, rank-quantised rows) are shared by all calls: an event recorded
+  // behind the kernels orders the next call after them when it comes on another stream (or on the runner's
+  // own), and re-packing, growing the buffers and deleting the runner wait for it on the host.
   void RunDeviceOnStream(const float *deviceInputs, void *deviceResults, int64_t rows, hipStream_t stream);
   // As RunDeviceOnStream, but the partial sums and rank-quantised rows go into the library's fixed
   // device array instead of allocated buffers: no allocation, no free, no synchronisation.  Throws when
@@ -97,6 +100,9 @@ private:
   void Release() noexcept;
   void RunHostChunk(const void *hostInputs, void *hostResults, int64_t rows);
   void InitDevice();
+  // Ordering of calls that share the runner's buffers (see RunDeviceOnStream).
+  void OrderAfterAsyncCall(hipStream_t stream); // device-side: `stream` waits for the last asynchronous call
+  void WaitForAsyncCall();                       // host-side: returns when the last asynchronous call has finished
   void UploadModel();
   void FreeModel();
   void EnsurePartial(int64_t rows);
@@ -107,8 +113,9 @@ private:
     double *partial = nullptr; // [PartialCount()][rows][max(1, classes)] when NeedsFinalize()
     uint8_t *ranks = nullptr;  // rank-quantised rows when the plan uses them
   };
-  // Allocating callers: grows the runner's own buffers to hold `rows` rows.
-  Workspace OwnWorkspace(int64_t rows);
+  // Allocating callers: grows the runner's own buffers to hold `rows` rows and orders `stream`, on which the
+  // caller is about to launch, behind an asynchronous call that may still use them.
+  Workspace OwnWorkspace(int64_t rows, hipStream_t stream);
   size_t PartialBytes(int64_t rows) const;
   size_t RanksBytes(int64_t rows) const;
   // Rank-quantised plans: runs the binning kernel and returns the buffer the walk kernel reads.
@@ -138,6 +145,9 @@ private:
   size_t m_pinnedBytes = 0;
   std::unique_ptr<ParallelCopier> m_copier;
   hipEvent_t m_evStart = nullptr, m_evStop = nullptr;
+  hipEvent_t m_asyncDone = nullptr; // recorded behind the kernels of the last RunDeviceOnStream call
+  hipStream_t m_asyncStream = nullptr;
+  bool m_asyncPending = false;
 
   DeviceGlobalNode *m_dGlobalNodes = nullptr;
   DeviceGlobalTree *m_dGlobalTrees = nullptr;

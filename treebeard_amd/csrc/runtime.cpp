@@ -415,6 +415,11 @@ int32_t tbmi_set_global_walk_plan(intptr_t h, int32_t rowsPerBlock, int32_t inte
         InferenceRunner *r = Runner(h);
         LaunchPlan plan;
         plan.kernel = LaunchPlan::Kernel::kGlobalWalk;
+        // what the options asked of the walk stays in the plan: a tiled runner is refused by the packer (the
+        // global-memory walk has scalar nodes only) instead of quietly turning into a scalar walk
+        plan.tileSize = r->Model().plan.tileSize;
+        plan.tiling = r->Model().plan.tiling;
+        plan.peelWalks = r->Model().plan.peelWalks;
         plan.rowsPerBlock = rowsPerBlock > 0 ? rowsPerBlock : 256;
         plan.interleave = interleave > 0 ? interleave : 4;
         plan.treeSlices = treeSlices > 0 ? treeSlices : 1;
@@ -491,6 +496,15 @@ intptr_t tbmi_load_compiled_model(const char *path, int32_t batchSize) {
         return reinterpret_cast<intptr_t>(new InferenceRunner(std::move(m.forest), options, m.plan, std::move(m.profile)));
       },
       0);
+}
+
+// src/runtime/runtime.cpp:35-54.  The reference reopens a compiled shared object together with the JSON of its
+// model buffers; here the compiled model is the one file tbmi_save_compiled_model writes, named by `soPath`, and
+// it holds everything the reference reads from the JSON (tile size, type widths, the model), so the second
+// path is not opened.
+intptr_t InitializeInferenceRunner(const char *soPath, const char *modelGlobalsJSONPath) {
+  (void)modelGlobalsJSONPath;
+  return tbmi_load_compiled_model(soPath, 0);
 }
 
 int32_t tbmi_forest_load_profile(intptr_t h, const char *profileCSVPath, int64_t *numRows, double *expectedSteps) {

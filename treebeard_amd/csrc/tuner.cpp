@@ -78,7 +78,12 @@ LaunchPlan ChooseTreeParallelPlan(const Forest &forest, int64_t batchSize, const
 
 namespace {
 LaunchPlan ChooseScalarPlan(const Forest &forest, int64_t batchSize, const GPUAutoScheduleOptions *ov,
-                            const DeviceLimits &limits, bool tiled);
+                            const DeviceLimits &limits, int tileSize);
+// LDS bytes a tree group must offer the biggest tree of a tiled forest (the null leaf tile and the alignment
+// pad of a group included).
+int64_t TiledGroupNeed(const Forest &forest, int tileSize) {
+  return BiggestTiledTreeBytes(forest, tileSize) + 2 * (int64_t)TileBytes(tileSize) + 16;
+}
 }
 
 LaunchPlan ChoosePlan(const Forest &forest, int64_t batchSize, const GPUAutoScheduleOptions *ov,
@@ -86,7 +91,7 @@ LaunchPlan ChoosePlan(const Forest &forest, int64_t batchSize, const GPUAutoSche
   if (walk.tileSize < 1 || walk.tileSize > kMaxTileSize)
     throw Error("tile size " + std::to_string(walk.tileSize) + " is not supported: the device kernels walk tiles of 1 to " +
                 std::to_string(kMaxTileSize) + " nodes");
-  LaunchPlan plan = ChooseScalarPlan(forest, batchSize, ov, limits, walk.tileSize > 1);
+  LaunchPlan plan = ChooseScalarPlan(forest, batchSize, ov, limits, walk.tileSize);
   plan.tileSize = walk.tileSize;
   plan.tiling = walk.tiling;
   plan.peelWalks = walk.peelWalks;
@@ -95,13 +100,14 @@ LaunchPlan ChoosePlan(const Forest &forest, int64_t batchSize, const GPUAutoSche
 
 namespace {
 
-// `tiled`: the plan must be the row-parallel kernel on f32 rows with byte offsets (tiles hold byte offsets
-// into a row tile below 64 KB), and groups are sized for tiles, which take about three times the bytes of
+// tileSize > 1: the plan must be the row-parallel kernel on f32 rows with byte offsets (tiles hold byte offsets
+// into a row tile below 64 KB), and groups are sized for tiles, which take three to eight times the bytes of
 // scalar nodes.
 LaunchPlan ChooseScalarPlan(const Forest &forest, int64_t batchSize, const GPUAutoScheduleOptions *ov,
-                            const DeviceLimits &limits, bool tiled) {
-  if (tiled) {
-    if ((BiggestTreeNodes(forest) + 2) * 32 > 65536)
+                            const DeviceLimits &limits, int tileSize) {
+  if (tileSize > 1) {
+    const int64_t need = TiledGroupNeed(forest, tileSize);
+    if (need > 65536)
       throw Error("tile sizes above 1 need every tree to fit one LDS tree group; this forest has a tree that does not");
     LaunchPlan plan;
     plan.kernel = LaunchPlan::Kernel::kRowParallelLds;
@@ -120,13 +126,12 @@ LaunchPlan ChooseScalarPlan(const Forest &forest, int64_t batchSize, const GPUAu
     const int64_t meet = forest.numClasses > 0 ? (int64_t)rb * plan.treeThreads * 8 : 0;
     int64_t budget = limits.ldsBytesPerBlock / 2;
     int64_t group = std::min<int64_t>(65536, budget - tileBytes(rb) - meet - 512);
-    const int64_t need = (BiggestTreeNodes(forest) + 2) * 32;
     if (group < need) group = std::min<int64_t>(65536, limits.ldsBytesPerBlock - tileBytes(rb) - meet - 512);
     group = std::min<int64_t>(group, 256LL * rb * plan.treeThreads);
     if (group < need) throw Error("the biggest tree does not fit LDS next to the row tile when tiled");
     plan.groupBytes = (int32_t)(group & ~15);
     const int64_t rowBlocks = std::max<int64_t>(1, (batchSize + rb - 1) / rb);
-    const int64_t totalBytes = (int64_t)forest.NumNodes() * 24;
+    const int64_t totalBytes = (int64_t)forest.NumNodes() * (tileSize > kMaxSelectTile ? 40 : 24);
     int64_t slices = 1;
     const int64_t wantBlocks = 2LL * limits.computeUnits;
     if (rowBlocks < wantBlocks) slices = (wantBlocks + rowBlocks - 1) / rowBlocks;
@@ -285,7 +290,7 @@ std::vector<LaunchPlan> CandidatePlans(const Forest &forest, int64_t batchSize, 
         if (tile > 0xFFFF) continue;
         const int64_t meet = forest.numClasses > 0 ? (int64_t)rb * p.treeThreads * 8 : 0;
         int64_t group = std::min<int64_t>(65536, limits.ldsBytesPerBlock / 2 - tile - meet - 2048);
-        if (group < (BiggestTreeNodes(forest) + 2) * 32) continue;
+        if (group < TiledGroupNeed(forest, base.tileSize)) continue;
         if (base.treeSlices > 1) group = std::min<int64_t>(group, base.groupBytes);
         p.groupBytes = (int32_t)(group & ~15);
         bool dup = false;

@@ -71,6 +71,7 @@ SIGNATURES = {
     "tbmi_describe_plan": (c_i32, [c_ip, c_cp, c_i32]),
     "tbmi_save_compiled_model": (c_i32, [c_ip, c_cp]),
     "tbmi_load_compiled_model": (c_ip, [c_cp, c_i32]),
+    "InitializeInferenceRunner": (c_ip, [c_cp, c_cp]),
     "tbmi_forest_load_profile": (c_i32, [c_ip, c_cp, ctypes.POINTER(c_i64), ctypes.POINTER(ctypes.c_double)]),
     "tbmi_num_trees": (c_i32, [c_ip]),
     "tbmi_num_classes": (c_i32, [c_ip]),

@@ -215,6 +215,13 @@ class TreebeardInferenceRunner:
             onnx_model_path.encode("ascii"), options.optionsPtr), "CreateInferenceRunnerForONNXModel"))
 
     @classmethod
+    def FromSOFile(cls, modelSOPath, modelGlobalsJSONPath=""):
+        """src/python/treebeard.py:314-319: reopens a compiled model through InitializeInferenceRunner.  Here
+        `modelSOPath` names a file written by save_compiled_model; the globals path is accepted and not opened."""
+        return cls._from_handle(_check(_lib().InitializeInferenceRunner(
+            modelSOPath.encode("ascii"), (modelGlobalsJSONPath or "").encode("ascii")), "InitializeInferenceRunner"))
+
+    @classmethod
     def FromCompiledModelFile(cls, path, batchSize=0):
         """Reopens a model saved with save_compiled_model (the counterpart of the reference's FromSOFile)."""
         return cls._from_handle(_check(_lib().tbmi_load_compiled_model(path.encode("ascii"), batchSize),
