@@ -513,7 +513,7 @@ def test_compiled_model_file_round_trip(synth_model, tmp_path, k):
     again = treebeard.TreebeardInferenceRunner.FromSOFile(path, str(tmp_path / "globals.json"))
     assert again.batchSize == rows and again.rowSize == forest.num_features and again.describe_plan() == plan
     check_against_oracle(again, forest, x)
-    np.testing.assert_array_equal(again.RunInference(x), expected)
+    np.testing.assert_array_equal(again.RunInference(x, again.result_dtype()), expected)
     with pytest.raises(RuntimeError, match="InitializeInferenceRunner"):
         treebeard.TreebeardInferenceRunner.FromSOFile(str(tmp_path / "missing.tbamd"), "")
     with open(path, "r+b") as fh:
@@ -1003,8 +1003,8 @@ def test_describe_plan_says_where_walk_peeling_applies(synth_model, tmp_path):
     forest = model_io.load_xgboost_json(synth_model(3))
     x = synth.CONFIGS[3].batch_rows(1000, seed_offset=3)
     profile = write_profile(tmp_path / "c3.profile.csv", forest, cpu_oracle.leaf_ids(forest, synth.CONFIGS[3].batch_rows(2000)))
-    runner = make_tiled_runner(synth_model(3), 1000, 1, 1, profile, True, multiclass=True)
-    assert " peelWalks=ignored(fused) " in runner.describe_plan()
+    runner = make_tiled_runner(synth_model(3), 1 << 17, 1, 1, profile, True, multiclass=True)   # (a batch that needs one tree slice)
+    assert " treeSlices=1 " in runner.describe_plan() and " peelWalks=ignored(fused) " in runner.describe_plan()
     check_against_oracle(runner, forest, x)
     runner.set_plan(128, 8, 4, 0, 2)                  # two tree slices: sums go through the finalize kernel
     assert " peelWalks=1 " in runner.describe_plan()
