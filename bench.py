@@ -45,6 +45,14 @@ def print_lds_read_costs():
                 print("| %s | %s | %s | %.2f |" % (name, pattern_name, mask_name, lds_read_cost(op, pattern, mask)), flush=True)
 
 
+def plan_key(plan):
+    """The fields of a plan description that decide which kernel runs and how (what a traffic figure is tied to)."""
+    keep = ("kernel", "rowsPerBlock", "treeThreads", "treeLanes", "interleave", "groupBytes", "treeSlices", "quantizedRows",
+            "tileSize", "staging")
+    fields = dict(item.split("=", 1) for item in plan.split() if "=" in item)
+    return " ".join("%s=%s" % (k, fields[k]) for k in keep if k in fields)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -56,7 +64,9 @@ def main():
     ap.add_argument("--group-staging", type=int, default=0, choices=[0, 1, 2],
                     help="how tree groups reach LDS: 0 by rule, 1 through prefetch registers, 2 direct global-to-LDS copies")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--autotune", action="store_true", help="timed launch-plan search before measuring")
+    ap.add_argument("--plan", choices=["tuned", "default"], default="tuned",
+                    help="tuned: the library's timed launch-plan search (what the reference's findBestGPUScheduleAndCompileModel "
+                         "stands for) picks the plan on this batch before anything is measured; default: the analytic plan")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU-baseline duration")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="also run one plain device copy of this many MiB (counter calibration for rocprofv3 --pmc)")
@@ -88,7 +98,11 @@ def main():
     multiclass = runner.num_classes() > 0
     dx = torch.from_numpy(x).cuda()
     out = torch.zeros(rows, dtype=torch.int8 if multiclass else torch.float32, device="cuda")
-    if args.autotune:
+    default_plan = runner.describe_plan()
+    default_plan_ms = None
+    if args.plan == "tuned":
+        runner.time_kernels3(dx.data_ptr(), out.data_ptr(), rows, 5)                     # (clocks ramp up)
+        default_plan_ms = sum(runner.time_kernels3(dx.data_ptr(), out.data_ptr(), rows, 10))
         runner.autotune(dx.data_ptr(), rows)
     if args.copy_calibration:
         # a plain device copy of known size: scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run
@@ -180,11 +194,17 @@ def main():
                      "frac_of_lockstep_floor": lockstep_ms / walk_ms}
     # HBM bytes per launch of the timed kernels, from rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this same command
     # (scaled by a plain copy of known size); read from the committed summary, not measured in this run
-    traffic = None
+    traffic, traffic_note = None, None
     traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(traffic_file):
         with open(traffic_file) as fh:
-            traffic = json.load(fh).get("%s@%d" % (cfg.name, rows), {}).get("bytes_per_launch")
+            entry = json.load(fh).get("%s@%d" % (cfg.name, rows), {})
+        # the counters were taken on one launch plan: a figure measured on another plan is not this run's traffic
+        if entry.get("plan") == plan_key(plan):
+            traffic = entry.get("bytes_per_launch")
+        elif entry:
+            traffic_note = ("profiles/hbm_traffic.json holds %.4g bytes per launch measured on plan [%s]; this run used [%s]"
+                            % (entry.get("bytes_per_launch", 0), entry.get("plan"), plan_key(plan)))
 
     # The roofline that binds this workload (the larger of the two times above): LDS node + feature reads for the
     # narrow models, HBM row streaming for the wide one.  `achieved` = algorithmic bytes per launch / the dominant
@@ -200,7 +220,7 @@ def main():
                              "instructions of about 2.5 clk each (measured), so about 50 % is its ceiling"}
     roofline = dict(lds_view if binding == "lds" else hbm_view)
     roofline.update({"traffic": traffic, "traffic_source": "profiles/hbm_traffic.json (rocprofv3 FETCH_SIZE + WRITE_SIZE "
-                                                           "of this command, scaled by a plain copy)" if traffic else None,
+                                                           "of this command, scaled by a plain copy)" if traffic else traffic_note,
                      "kernel": ("BinRowsKernel+" if quantized else "") + kernel,
                      "kernel_ms": hbm_ms if binding == "hbm" else walk_ms,
                      "walk_ms": walk_ms, "finalize_ms": fin_ms, "bin_ms": bin_ms, "path_ms": path_ms})
@@ -211,7 +231,9 @@ def main():
         "ms_per_step": ms_per_step, "ms_per_step_sync_every_call": ms_per_step_sync, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": cfg.name, "rows": rows, "trees": forest.num_trees, "features": cfg.num_features,
-                   "objective": cfg.objective, "plan": plan},
+                   "objective": cfg.objective, "plan": plan,
+                   "plan_source": "timed search over launch plans on this batch (tbmi_autotune)" if args.plan == "tuned"
+                   else "analytic default", "default_plan": default_plan, "default_plan_path_ms": default_plan_ms},
         "roofline": roofline,
         "roofline_other": hbm_view if binding == "lds" else lds_view,   # the memory roofline that does not bind
     }

@@ -178,6 +178,13 @@ TBAMD_EXPORT int32_t tbmi_set_global_walk_plan(intptr_t runner, int32_t rowsPerB
 /* Pins the row-parallel kernel on rank-quantised rows (64 rows per block, one byte per feature value). */
 TBAMD_EXPORT int32_t tbmi_set_quantized_plan(intptr_t runner, int32_t treeThreads, int32_t interleave,
                                              int32_t groupBytes, int32_t treeSlices);
+/* Pins the row-parallel kernel on two-byte rank rows: a ranking kernel first replaces every value by the number
+ * of its feature's distinct split thresholds that are <= it (exact: every comparison keeps its outcome), laid
+ * out so that the walk's row tile takes half the LDS of float32 rows.  For models of up to about 120 features
+ * (the tile of `rowsPerBlock` rows must stay below 64 KB) with at most 65534 distinct thresholds per feature.
+ * No counterpart in the reference. */
+TBAMD_EXPORT int32_t tbmi_set_rank16_plan(intptr_t runner, int32_t rowsPerBlock, int32_t treeThreads, int32_t interleave,
+                                          int32_t groupBytes, int32_t treeSlices);
 /* How the row-parallel scalar walk brings tree groups into LDS: 0 by rule (direct global-to-LDS copies when two
  * blocks fit a compute unit, through prefetch registers otherwise), 1 always through registers, 2 always direct.
  * Results do not depend on it.  No counterpart in the reference (its GPU schedules cache trees with cooperative

@@ -148,7 +148,9 @@ uint32_t Bits(float v) {
 
 // One row through the slice's groups of an LDS-layout model.  `stride` is the node-offset distance between
 // two features; rankRows: x points at the rank tile [row block][feature][64 rows].
-void WalkRowLds(const WalkParams &p, int K, uint32_t stride, bool rankRows, int64_t row, int slice, double *classSums,
+// rankRows: 0 f32 rows, 1 one-byte ranks, 2 two-byte ranks ([row block][feature pair][row][2], `stride` = bytes of
+// one feature pair's column = rows per block x 4)
+void WalkRowLds(const WalkParams &p, int K, uint32_t stride, int rankRows, int64_t row, int slice, double *classSums,
                 bool *classSeen) {
   const DeviceNode *nodes = reinterpret_cast<const DeviceNode *>(p.nodes16);
   const int F = p.s.numFeatures;
@@ -163,10 +165,16 @@ void WalkRowLds(const WalkParams &p, int K, uint32_t stride, bool rankRows, int6
         for (uint32_t d = 0; d < bd.depth; ++d) {
           if (addr % kNodeBytes != 0 || addr / kNodeBytes >= grp.nodeCount) std::abort(); // pointer outside the group
           const DeviceNode node = nodes[grp.nodeBegin + addr / kNodeBytes];
-          const uint32_t f = (node.meta & 0xFFFFu) / stride;
-          if ((node.meta & 0xFFFFu) % stride != 0 || (int)f > F) std::abort(); // offset outside the row tile
+          const uint32_t offset = node.meta & 0xFFFFu;
+          const uint32_t f = rankRows == 2 ? offset / stride * 2u + ((offset >> 1) & 1u) : offset / stride;
+          if ((rankRows == 2 ? (offset % stride) & ~2u : offset % stride) != 0 || (int)f > F) std::abort(); // offset outside the row tile
           bool left;
-          if (rankRows) {
+          if (rankRows == 2) {
+            const uint16_t *ranks = reinterpret_cast<const uint16_t *>(p.x);
+            const int64_t RB = stride / 4, pairs = (F + 2) / 2;
+            const uint32_t rank = ranks[(((row / RB) * pairs + f / 2) * RB + row % RB) * 2 + (f & 1)]; // (the pad feature's slot holds 0)
+            left = rank <= Bits(node.value);
+          } else if (rankRows) {
             const uint8_t *ranks = reinterpret_cast<const uint8_t *>(p.x);
             const uint32_t rank = (int)f == F ? 0u : ranks[((row / 64) * F + f) * 64 + (row % 64)];
             left = rank <= Bits(node.value);
@@ -213,7 +221,7 @@ void StoreRow(const WalkParams &p, int64_t row, int slice, const double *classSu
   }
 }
 
-hipError_t WalkLds(const WalkParams &p, int K, uint32_t stride, bool rankRows) {
+hipError_t WalkLds(const WalkParams &p, int K, uint32_t stride, int rankRows) {
   if (K != 1 && K != 2 && K != 4 && K != 8) return hipErrorInvalidValue;
   if (p.s.treeSlices > 1 && !p.partial) std::abort(); // slices meet in the partial-sum buffer
   const int Cn = p.s.numClasses > 0 ? p.s.numClasses : 1;
@@ -238,9 +246,10 @@ hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, int tileMode, 
   const int prefetch = (int)((p.s.groupRegionBytes / 16 + RB * TT - 1) / (RB * TT));
   if (prefetch > 16) return hipErrorInvalidValue;
   if (tileMode == 2 && RB != 64) return hipErrorInvalidValue;
-  if (tileMode < 0 || tileMode > 2) return hipErrorInvalidValue;
-  const uint32_t stride = tileMode == 0 ? (uint32_t)RB * 4u : tileMode == 1 ? (uint32_t)RB : (uint32_t)RB / 4u;
-  return WalkLds(p, interleave, stride, tileMode == 2);
+  if (tileMode < 0 || tileMode > 3) return hipErrorInvalidValue;
+  if (tileMode == 3 && (int64_t)((p.s.numFeatures + 2) / 2) * RB * 4 > 0x10000) return hipErrorInvalidValue;
+  const uint32_t stride = tileMode == 0 || tileMode == 3 ? (uint32_t)RB * 4u : tileMode == 1 ? (uint32_t)RB : (uint32_t)RB / 4u;
+  return WalkLds(p, interleave, stride, tileMode == 3 ? 2 : tileMode == 2 ? 1 : 0);
 }
 
 namespace {
@@ -355,7 +364,7 @@ hipError_t LaunchWalkTreeParallel(const WalkParams &p, int interleave, size_t ld
   if (threads > 1024 || threads % 64 != 0) return hipErrorInvalidValue;
   if (p.s.treeSlices < 1 || p.s.treeSlices > 65535) return hipErrorInvalidValue;
   if ((int)((p.s.groupRegionBytes / 16 + threads - 1) / threads) > 16) return hipErrorInvalidValue;
-  return WalkLds(p, interleave, 4u, false);
+  return WalkLds(p, interleave, 4u, 0);
 }
 
 hipError_t LaunchWalkGlobal(const WalkParams &p, int interleave, hipStream_t) {
@@ -403,6 +412,45 @@ hipError_t LaunchBinRows(const float *x, const float *table, uint8_t *ranks, int
           if (!(v < column[(int64_t)(rank + step - 1) * 64])) rank += step;
         ranks[(rb * numFeatures + f) * 64 + r] = (uint8_t)rank;
       }
+  return hipSuccess;
+}
+
+hipError_t LaunchRankRows16(const float *x, const float *tables, const RankFeatureDesc *features, const RankChunkDesc *chunks,
+                            int numChunks, uint32_t maxChunkEntries, uint32_t maxChunkFeatures, uint16_t *ranks, int64_t rows,
+                            int numFeatures, int rowsPerBlock, hipStream_t) {
+  if (rows <= 0) return hipSuccess;
+  if (numChunks < 1 || (size_t)maxChunkEntries * 4 + (size_t)maxChunkFeatures * 1025 * 4 + 16 > 160 * 1024 || rowsPerBlock < 64 ||
+      rowsPerBlock % 64 != 0)
+    return hipErrorInvalidValue;
+  const int64_t RB = rowsPerBlock, pairs = (numFeatures + 2) / 2;
+  // the kernel ranks whole row blocks, rounded up to its own tiles of 1024 rows: the buffer has to hold them
+  const int64_t rowBlocks = (((rows + RB - 1) / RB * RB + 1023) / 1024 * 1024 + RB - 1) / RB;
+  std::vector<char> written((size_t)pairs * 2, 0);
+  for (int c = 0; c < numChunks; ++c) {
+    const RankChunkDesc ck = chunks[c];
+    if (ck.firstFeature % 2 || ck.numFeatures % 2 || ck.firstFeature + ck.numFeatures > (uint32_t)pairs * 2 ||
+        ck.tableEntries > maxChunkEntries || ck.numFeatures > maxChunkFeatures)
+      std::abort();
+    for (uint32_t f = ck.firstFeature; f < ck.firstFeature + ck.numFeatures; ++f) {
+      written[f] = 1;
+      const RankFeatureDesc fd = features[f];
+      const uint32_t entries = (1u << fd.levels) - 1u;
+      if (fd.tableOffset + entries > ck.tableEntries) std::abort(); // table outside its chunk
+      if ((int)f >= numFeatures && fd.levels != 0) std::abort();     // the pad slots have no table
+      const float *table = tables + ck.tableBegin + fd.tableOffset;
+      for (int64_t slot = 0; slot < rowBlocks * RB; ++slot) {
+        const int64_t row = std::min<int64_t>(slot, rows - 1);
+        uint32_t node = 0;
+        if (fd.levels) {
+          const float v = x[row * numFeatures + f];
+          for (uint32_t level = 0; level < fd.levels; ++level) node = 2 * node + (v < table[node] ? 1u : 2u);
+        }
+        ranks[(((slot / RB) * pairs + f / 2) * RB + slot % RB) * 2 + (f & 1)] = (uint16_t)(node - entries);
+      }
+    }
+  }
+  for (char w : written)
+    if (!w) std::abort(); // a slot of the tile no chunk fills
   return hipSuccess;
 }
 

@@ -295,6 +295,9 @@ void DeviceEntryPoints(const Case &c, int64_t rows, int32_t tileSize = 1, int32_
   const int quantized[][4] = {{8, 4, 0, 1}, {16, 1, 16384, 1}, {4, 2, 32768, 3}, {1, 8, 16384, 1}};
   for (auto &p : quantized)
     if (tbmi_set_quantized_plan(runner, p[0], p[1], p[2], p[3]) == 0) runAll("rank-quantised plan");
+  const int rank16[][5] = {{256, 4, 4, 0, 1}, {512, 2, 4, 32768, 1}, {128, 8, 2, 16384, 3}, {64, 1, 1, 16384, 2}};
+  for (auto &p : rank16)
+    if (tbmi_set_rank16_plan(runner, p[0], p[1], p[2], p[3], p[4]) == 0) runAll("two-byte rank plan");
   if (tbmi_set_global_walk_plan(runner, 256, 4, 3) == 0) runAll("global walk plan");
   double best = 0;
   EXPECT(tbmi_autotune(runner, dx, rows, &best) == 0, "tbmi_autotune");

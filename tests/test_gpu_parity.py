@@ -368,6 +368,60 @@ def test_rank_quantised_plans_agree(synth_model, tmp_path, model, plan):
     check_against_oracle(runner, forest, x)
 
 
+@pytest.mark.parametrize("plan", [(256, 4, 4, 0, 1), (512, 2, 4, 32768, 1), (128, 8, 2, 16384, 3), (64, 1, 1, 16384, 2), (1024, 1, 8, 16384, 1)])
+@pytest.mark.parametrize("model", ["config2", "config3", "config5", "coarse_regression", "coarse_multiclass"])
+def test_two_byte_rank_plans_agree(synth_model, tmp_path, model, plan):
+    """Rows replaced by two-byte ranks among each feature's thresholds (a ranking kernel in front of the walk, tile
+    [feature pair][row][2]): leaf selection must not change - even and odd feature counts, values that sit on
+    thresholds, +-inf and NaN, regressors and classifiers, several block shapes and tree slices."""
+    if model.startswith("config"):
+        k = int(model[-1])
+        path, rows = synth_model(k), 2500
+        x = synth.CONFIGS[k].batch_rows(rows, seed_offset=5)
+    else:
+        path, rows = str(tmp_path / "coarse.json"), 1500
+        coarse_model(path, 37, 120, 5 if model == "coarse_multiclass" else 0, seed=17)       # 37 features: the pad slot shares the last pair
+        rng = np.random.default_rng(3)
+        x = np.round(rng.normal(size=(rows, 37)), 2).astype(np.float32)     # many values equal to thresholds
+    forest = model_io.load_xgboost_json(path)
+    thr, feat, left, _ = forest.tree(0)
+    for i in np.nonzero(left != -1)[0][:20]:
+        x[int(i) % rows, feat[i]] = np.float32(thr[i])
+        x[(int(i) + 50) % rows, feat[i]] = np.nextafter(np.float32(thr[i]), np.float32(-np.inf))
+    x[3, :] = np.inf
+    x[4, :] = -np.inf
+    x[5, ::2] = np.nan
+    runner = make_runner(path, rows)
+    if plan[0] * ((forest.num_features + 2) // 2) * 4 > 65536:
+        with pytest.raises(RuntimeError, match="below 64 KB|do not fit 16 bits"):
+            runner.set_rank16_plan(*plan)
+        return
+    runner.set_rank16_plan(*plan)
+    assert "rankRows16=1" in runner.describe_plan() and "staging=direct" in runner.describe_plan()
+    check_against_oracle(runner, forest, x)
+    # the other entry points on the same plan: host buffers, the caller's stream, no allocation
+    expected = gpu_predict(runner, x)
+    np.testing.assert_array_equal(runner.RunInference(x, runner.result_dtype()), expected)
+    dx = torch.from_numpy(x).cuda()
+    got = torch.zeros(rows, dtype=torch.int8 if runner.result_dtype() == np.int8 else torch.float32, device="cuda")
+    stream = torch.cuda.current_stream()
+    runner.run_device_noalloc(dx.data_ptr(), got.data_ptr(), rows, stream.cuda_stream)
+    stream.synchronize()
+    np.testing.assert_array_equal(got.cpu().numpy(), expected)
+
+
+def test_two_byte_rank_plan_survives_the_compiled_model_file(synth_model, tmp_path):
+    forest = model_io.load_xgboost_json(synth_model(5))
+    x = synth.CONFIGS[5].batch_rows(3000, seed_offset=2)
+    runner = make_runner(synth_model(5), 3000)
+    runner.set_rank16_plan(256, 4, 8, 32768, 1)
+    path = str(tmp_path / "rank16.tbamd")
+    runner.save_compiled_model(path)
+    again = treebeard.TreebeardInferenceRunner.FromSOFile(path, "")
+    assert again.describe_plan() == runner.describe_plan() and "rankRows16=1" in again.describe_plan()
+    check_against_oracle(again, forest, x)
+
+
 def test_rank_quantisation_is_refused_when_a_feature_has_too_many_thresholds(synth_model):
     runner = make_runner(synth_model(2), 512)
     with pytest.raises(RuntimeError, match="254 distinct thresholds"):
@@ -821,9 +875,12 @@ def test_random_forests_and_plans(tmp_path, seed):
     runner = make_runner(path, rows, gpu_options=gpu)
     runner.set_group_staging(int(rng.integers(0, 3)))     # tree groups by rule, through registers, or copied directly
     check_against_oracle(runner, forest, x)
-    kind = rng.integers(0, 4)
+    kind = rng.integers(0, 5)
     try:
-        if kind == 0:
+        if kind == 4:
+            rb = int(rng.choice([64, 128, 256, 512]))
+            runner.set_rank16_plan(rb, int(rng.choice([1, 2, 1024 // rb])), int(rng.choice([1, 2, 4, 8])), 0, int(rng.integers(0, 5)))
+        elif kind == 0:
             runner.set_global_walk_plan(int(rng.choice([64, 256, 1024])), int(rng.choice([1, 2, 4, 8])), int(rng.integers(1, 50)))
         elif kind == 1:
             runner.set_quantized_plan(int(rng.choice([1, 4, 16])), int(rng.choice([1, 2, 4])), 0, int(rng.integers(1, 6)))

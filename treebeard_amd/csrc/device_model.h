@@ -102,6 +102,17 @@ struct DeviceGlobalTree {
   int32_t origin;     // tree index in the model file
 };
 
+// Ranking kernel of the two-byte rank rows: where a feature's threshold table (a complete search tree in
+// breadth-first order, 2^levels - 1 entries) starts inside its chunk, and which whole feature pairs a chunk holds.
+struct RankFeatureDesc {
+  uint32_t tableOffset;
+  uint32_t levels;
+};
+struct RankChunkDesc {
+  uint32_t firstFeature, numFeatures;
+  uint32_t tableBegin, tableEntries;
+};
+
 struct DeviceGroup {
   uint32_t nodeBegin;   // first node of the group in the packed node array
   uint32_t nodeCount;   // multiple of 2 so that the group is a whole number of 16-byte pieces

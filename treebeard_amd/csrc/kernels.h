@@ -67,7 +67,8 @@ struct FinalizeParams {
 
 // Row-parallel walk over LDS-staged tree groups: block = s.rowsPerBlock * s.treeThreads lanes.
 // `interleave` in {1,2,4,8}; `tileMode`: 0 f32 tile with byte offsets, 1 f32 tile with offsets in units of
-// 4 bytes, 2 one-byte rank tile (p.x then points at the output of LaunchBinRows; 64 rows per block).
+// 4 bytes, 2 one-byte rank tile (p.x then points at the output of LaunchBinRows; 64 rows per block), 3 two-byte
+// rank tile (p.x points at the output of LaunchRankRows16 for the same rowsPerBlock).
 hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, int tileMode, size_t ldsBytes, hipStream_t stream);
 // The same block shape over tiled trees (tiles of 2 to 8 nodes, f32 row tile with byte offsets below 64 KB);
 // `interleave` in {1,2,4}.  Tree groups are staged by direct global-to-LDS copies.
@@ -76,6 +77,13 @@ hipError_t LaunchWalkRowsTiled(const WalkParams &p, int tileSize, int interleave
 // packer's threshold table ([chunk][k][64], +inf padded, tableDepth = 2^n - 1).
 hipError_t LaunchBinRows(const float *x, const float *table, uint8_t *ranks, int64_t rows, int numFeatures,
                          int tableDepth, int chunkFeatures, hipStream_t stream);
+// Ranks rows x[rows][numFeatures] into two-byte ranks laid out as [ceil(rows / rowsPerBlock)][(numFeatures + 2) / 2]
+// [rowsPerBlock][2] with the packer's tables (PackedModel::rankTables / rankFeatures / rankChunks on the device);
+// maxChunkEntries / maxChunkFeatures = the largest chunk's table entries / slots (the kernel's LDS need).  The rank
+// buffer must hold the rows rounded up to whole row blocks and then to a multiple of 1024 rows.
+hipError_t LaunchRankRows16(const float *x, const float *tables, const RankFeatureDesc *features, const RankChunkDesc *chunks,
+                            int numChunks, uint32_t maxChunkEntries, uint32_t maxChunkFeatures, uint16_t *ranks, int64_t rows,
+                            int numFeatures, int rowsPerBlock, hipStream_t stream);
 // Tree-parallel walk: s.rowsPerBlock rows per block (row-major in LDS),
 // s.treeLanes lanes per row; block = rowsPerBlock * treeLanes lanes.
 hipError_t LaunchWalkTreeParallel(const WalkParams &p, int interleave, size_t ldsBytes, hipStream_t stream);

@@ -27,13 +27,23 @@ __device__ __forceinline__ U32x2 LdsLoadNode(uint32_t address) { return *(LdsNod
 __device__ __forceinline__ float LdsLoadFloat(uint32_t address) { return *(LdsFloatPtr)(uintptr_t)address; }
 typedef const __attribute__((address_space(3))) uint8_t *LdsBytePtr;
 __device__ __forceinline__ uint32_t LdsLoadByte(uint32_t address) { return *(LdsBytePtr)(uintptr_t)address; }
+typedef const __attribute__((address_space(3))) uint16_t *LdsHalfPtr;
+__device__ __forceinline__ uint32_t LdsLoadHalf(uint32_t address) { return *(LdsHalfPtr)(uintptr_t)address; }
 
 // How a node's 16-bit feature offset addresses the row tile of the row-parallel kernel.
 enum RowTileMode : int {
   kTileF32Bytes = 0, // f32 tile, offset in bytes
   kTileF32Words = 1, // f32 tile, offset in units of 4 bytes (tiles above 64 KB)
-  kTileRankU8 = 2    // one-byte rank tile (rank-quantised rows), offset in units of 4 bytes
+  kTileRankU8 = 2,   // one-byte rank tile (rank-quantised rows), offset in units of 4 bytes
+  kTileRankU16 = 3   // two-byte rank tile [feature pair][row][2], offset in bytes
 };
+constexpr bool IsRankTile(int mode) { return mode == kTileRankU8 || mode == kTileRankU16; }
+
+// A rank tile's comparison: the row's rank among the feature's thresholds against the node's threshold index.
+template <int kMode>
+__device__ __forceinline__ bool RankGoesLeft(uint32_t address, uint32_t thresholdIndex) {
+  return (kMode == kTileRankU8 ? LdsLoadByte(address) : LdsLoadHalf(address)) <= thresholdIndex;
+}
 
 
 // Copies the block's rows (contiguous, row-major in global memory) into the LDS tile.
@@ -149,12 +159,14 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
   const int valid = remaining < RB ? (int)remaining : RB;
 
   uint32_t column; // LDS address of this row's feature 0
-  if (kMode == kTileRankU8) {
-    // Rank-quantised rows arrive already tiled ([row block][feature][row], one byte each): plain copy.
+  if (IsRankTile(kMode)) {
+    // Ranks arrive already tiled: plain copy.  One byte each as [row block][feature][row] (the pad feature's
+    // column is filled here), or two bytes each as [row block][feature pair][row][2], pad feature included.
     typedef uint32_t Piece __attribute__((ext_vector_type(4)));
-    const Piece *src = reinterpret_cast<const Piece *>(reinterpret_cast<const uint8_t *>(x) + (int64_t)blockIdx.x * F * RB);
+    const int tileBytes = kMode == kTileRankU8 ? F * RB : ((F + 2) >> 1) * RB * 4;
+    const Piece *src = reinterpret_cast<const Piece *>(reinterpret_cast<const uint8_t *>(x) + (int64_t)blockIdx.x * tileBytes);
     Piece *dst = reinterpret_cast<Piece *>(lds + s.groupRegionBytes);
-    const int pieces = (F * RB) >> 4;
+    const int pieces = tileBytes >> 4;
     for (int base = 0; base < pieces; base += threads * kStageUnroll) {
       Piece v[kStageUnroll];
 #pragma unroll
@@ -168,8 +180,12 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
         if (idx < pieces) dst[idx] = v[u];
       }
     }
-    for (int i = tid; i < RB; i += threads) lds[s.groupRegionBytes + (uint32_t)F * RB + i] = 0; // pad feature: rank 0
-    column = s.groupRegionBytes + (uint32_t)lane;
+    if (kMode == kTileRankU8) {
+      for (int i = tid; i < RB; i += threads) lds[s.groupRegionBytes + (uint32_t)F * RB + i] = 0; // pad feature: rank 0
+      column = s.groupRegionBytes + (uint32_t)lane;
+    } else {
+      column = s.groupRegionBytes + (uint32_t)lane * 4u;
+    }
   } else {
     float *rowTile = reinterpret_cast<float *>(lds + s.groupRegionBytes);
     // Stage the block's rows: coalesced reads of the contiguous row-major tile, transposed writes.
@@ -188,7 +204,9 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
   // them in thread order.  Classifiers meet at class boundaries, while a tree group is live, so
   // their meeting area sits behind the row tile; otherwise the (then idle) group region is used.
   double *meet = reinterpret_cast<double *>(
-      C > 0 ? lds + ((s.groupRegionBytes + (uint32_t)(F + 1) * RB * (kMode == kTileRankU8 ? 1u : 4u) + 7u) & ~7u) : lds);
+      C > 0 ? lds + ((s.groupRegionBytes + (kMode == kTileRankU16 ? (uint32_t)((F + 2) >> 1) * RB * 4u
+                                                                  : (uint32_t)(F + 1) * RB * (kMode == kTileRankU8 ? 1u : 4u)) + 7u) & ~7u)
+            : lds);
 
   double acc = 0.0;
   int curClass = 0;
@@ -299,8 +317,10 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
 #pragma unroll
           for (int k = 0; k < K; ++k) {
             const DeviceNode root = roots[k];
-            const uint32_t off = kMode == kTileF32Bytes ? (root.meta & 0xFFFFu) : (root.meta & 0xFFFFu) << 2;
-            const bool left = LdsLoadFloat(column + off) < root.value;
+            const uint32_t off = kMode == kTileF32Words ? (root.meta & 0xFFFFu) << 2 : (root.meta & 0xFFFFu);
+            bool left;
+            if (kMode == kTileRankU16) left = RankGoesLeft<kMode>(column + off, __float_as_uint(root.value));
+            else left = LdsLoadFloat(column + off) < root.value;
             addr[k] = (root.meta >> 16) + (left ? 0u : kNodeBytes);
           }
         }
@@ -310,9 +330,9 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
 #pragma unroll
           for (int k = 0; k < K; ++k) {
             const U32x2 node = LdsLoadNode(addr[k]);
-            const uint32_t off = kMode == kTileF32Bytes ? (node.y & 0xFFFFu) : (node.y & 0xFFFFu) << 2;
+            const uint32_t off = kMode == kTileF32Bytes || kMode == kTileRankU16 ? (node.y & 0xFFFFu) : (node.y & 0xFFFFu) << 2;
             bool left;
-            if (kMode == kTileRankU8) left = LdsLoadByte(column + off) <= node.x; // rank <= threshold index
+            if (IsRankTile(kMode)) left = RankGoesLeft<kMode>(column + off, node.x); // rank <= threshold index
             else left = LdsLoadFloat(column + off) < AsFloat(node.x);
             addr[k] = (node.y >> 16) + (left ? 0u : kNodeBytes);
           }
@@ -323,9 +343,9 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
 #pragma unroll
             for (int k = 0; k < K; ++k) {
               const U32x2 node = LdsLoadNode(addr[k]);
-              const uint32_t off = kMode == kTileF32Bytes ? (node.y & 0xFFFFu) : (node.y & 0xFFFFu) << 2;
+              const uint32_t off = kMode == kTileF32Bytes || kMode == kTileRankU16 ? (node.y & 0xFFFFu) : (node.y & 0xFFFFu) << 2;
               bool left;
-              if (kMode == kTileRankU8) left = LdsLoadByte(column + off) <= node.x;
+              if (IsRankTile(kMode)) left = RankGoesLeft<kMode>(column + off, node.x);
               else left = LdsLoadFloat(column + off) < AsFloat(node.x);
               const uint32_t next = (node.y >> 16) + (left ? 0u : kNodeBytes);
               moved = moved || next != addr[k];
@@ -978,6 +998,130 @@ BinRowsKernel(const float *__restrict__ x, const float *__restrict__ table, uint
 }
 
 // ---------------------------------------------------------------------------
+// Two-byte ranks for narrow models.  For every (row, feature) the kernel counts how many of the feature's
+// sorted distinct split thresholds are <= the value and writes the count as 16 bits into the tile layout the
+// row-parallel kernel copies verbatim: [block of RB rows][feature pair][row][2] (the two ranks of a pair share
+// a dword, so a row's LDS column keeps one bank of its own).  NaN and +inf count every entry of the table (a
+// rank above every node's threshold index: they go right at every node, as the f32 compare sends them).  The
+// slots of the pad feature (and of the unused half of an odd last pair) get rank 0.
+//
+// A block owns one chunk of feature pairs, whose threshold tables sit in LDS, and a range of rows, which it
+// takes 1024 at a time: the chunk's columns of those rows are read with row-contiguous loads and left
+// transposed in LDS (a lane that walked its row's columns in global memory would touch a cache line per load
+// and evict it before the next: measured 1.2 to 2 times slower), then a lane is a row: it picks its values out
+// of its own LDS bank and searches one feature after the other.  Every table is a complete search tree in
+// breadth-first order (entry 0 the root, then its children, ...) and the feature is the same for the whole
+// wave, so at search step l the lanes read among 2^l neighbouring entries (one bank each up to 64, broadcast
+// where they meet).  Blocks 8 apart in launch order (same XCD, back to back) take the chunks of one row range,
+// so that the cache lines of a row, which the chunks share, are fetched from HBM once.
+// ---------------------------------------------------------------------------
+// (measured on configurations 2, 3 and 5 at 2^20 rows: 16 waves x 1 group 0.105 / 0.169 / 0.290 ms, 8 x 2 0.120 / 0.189 /
+// 0.310, 4 x 4 0.152 / 0.252 / 0.365: the two phases of a tile are latency-bound, and waves hide latency better
+// than chains do)
+constexpr int kRankWaves = 16;
+constexpr int kRankChains = 1;                              // 64-row groups a lane searches side by side
+constexpr int kRankTileRows = kRankWaves * kRankChains * 64; // rows a block ranks between two barriers
+constexpr int kRankStride = kRankTileRows + 1;              // floats per feature column of the staging tile
+constexpr int kRankLoads = 8;                               // loads a lane keeps in flight while staging
+
+__global__ void __launch_bounds__(kRankWaves * 64)
+RankRows16Kernel(const float *__restrict__ x, const float *__restrict__ tables, const RankFeatureDesc *__restrict__ features,
+                 const RankChunkDesc *__restrict__ chunks, uint32_t *__restrict__ ranks, int64_t rows, int F, int RB,
+                 int numChunks, int tilesPerBlock, int64_t rowTiles, uint32_t tableRegionBytes) {
+  extern __shared__ __align__(16) unsigned char lds[];
+  const uint32_t linear = blockIdx.x;
+  const int chunk = (int)((linear >> 3) % (uint32_t)numChunks);
+  const int64_t range = (int64_t)(linear & 7u) + 8 * (int64_t)(linear / (8u * (uint32_t)numChunks));
+  const RankChunkDesc ck = chunks[chunk];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  constexpr int threads = kRankWaves * 64;
+  {
+    float *tab = reinterpret_cast<float *>(lds);
+    const float *src = tables + ck.tableBegin;
+    for (uint32_t i = tid; i < ck.tableEntries; i += threads) tab[i] = src[i];
+  }
+  float *stage = reinterpret_cast<float *>(lds + tableRegionBytes); // [feature of the chunk][kRankStride]
+  const uint32_t stageAddress = tableRegionBytes;
+  const int pairsTotal = (F + 2) >> 1;
+  const int Fc = (int)ck.numFeatures;                                // slots of the chunk (whole pairs)
+  const int live = (int)ck.firstFeature + Fc <= F ? Fc : F - (int)ck.firstFeature; // of which real features (may be <= 0)
+  const float invLive = live > 0 ? 1.0f / (float)live : 0.0f;
+  const int64_t tBegin = range * tilesPerBlock; // (past the end for the padding blocks of the last 8 ranges)
+  const int64_t tEnd = tBegin + tilesPerBlock < rowTiles ? tBegin + tilesPerBlock : rowTiles;
+  for (int64_t tile = tBegin; tile < tEnd; ++tile) {
+    const int64_t row0 = tile * kRankTileRows;
+    __syncthreads(); // tables loaded / the staging tile is no longer read
+    // The chunk's columns of the tile's rows: element e = (row, column) in row-major order, so that a wave's load
+    // covers whole row segments; rows past the batch (padding of the last row block) take the last row's values.
+    const int total = kRankTileRows * live;
+    for (int e0 = tid; e0 < total; e0 += threads * kRankLoads) {
+      float value[kRankLoads];
+      int where[kRankLoads];
+#pragma unroll
+      for (int u = 0; u < kRankLoads; ++u) {
+        const int e = e0 + u * threads < total ? e0 + u * threads : total - 1;
+        int r = (int)((float)e * invLive);
+        if (r * live > e) --r;
+        if ((r + 1) * live <= e) ++r;
+        const int j = e - r * live;
+        const int64_t row = row0 + r < rows ? row0 + r : rows - 1;
+        value[u] = x[row * F + ck.firstFeature + j];
+        where[u] = j * kRankStride + r;
+      }
+#pragma unroll
+      for (int u = 0; u < kRankLoads; ++u)
+        if (e0 + u * threads < total) stage[where[u]] = value[u];
+    }
+    __syncthreads();
+    // a lane is a row in each of its wave's kRankChains groups of 64 rows
+    const int r0 = wave * (kRankChains * 64) + lane;
+    int64_t slot[kRankChains];
+#pragma unroll
+    for (int c = 0; c < kRankChains; ++c) {
+      const int64_t row = row0 + r0 + c * 64;
+      slot[c] = (row / RB) * (int64_t)pairsTotal * RB + (row % RB) + (int64_t)(ck.firstFeature >> 1) * RB;
+    }
+    for (int j0 = 0; j0 < Fc; j0 += 2) {
+      uint32_t rank[2][kRankChains];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int j = j0 + h;
+        if (j >= live) { // the pad feature's slot and the unused half of an odd last pair
+#pragma unroll
+          for (int c = 0; c < kRankChains; ++c) rank[h][c] = 0;
+          continue;
+        }
+        const RankFeatureDesc fd = features[ck.firstFeature + j]; // (the same for the whole wave)
+        const uint32_t base = fd.tableOffset * 4u;                 // LDS byte address of the table's root
+        const uint32_t goLeft = 4u - base, goRight = 8u - base;
+        float v[kRankChains];
+        uint32_t pos[kRankChains];
+#pragma unroll
+        for (int c = 0; c < kRankChains; ++c) {
+          v[c] = LdsLoadFloat(stageAddress + (uint32_t)(j * kRankStride + r0 + c * 64) * 4u);
+          pos[c] = base;
+        }
+        for (uint32_t level = 0; level < fd.levels; ++level) {
+          float probe[kRankChains];
+#pragma unroll
+          for (int c = 0; c < kRankChains; ++c) probe[c] = LdsLoadFloat(pos[c]);
+#pragma unroll
+          for (int c = 0; c < kRankChains; ++c) pos[c] = (pos[c] << 1) + (v[c] < probe[c] ? goLeft : goRight); // NaN: right at every step
+        }
+        // entry index reached below the last table level, minus the 2^levels - 1 entries of the table = thresholds <= value
+        const uint32_t entries = (1u << fd.levels) - 1u;
+#pragma unroll
+        for (int c = 0; c < kRankChains; ++c) rank[h][c] = ((pos[c] - base) >> 2) - entries;
+      }
+#pragma unroll
+      for (int c = 0; c < kRankChains; ++c) ranks[slot[c] + (int64_t)(j0 >> 1) * RB] = rank[0][c] | (rank[1][c] << 16);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Sums the tree-slice partials of each row (in slice order, starting from the
 // initial value), then applies the output transform.  Multiclass rows get the
 // arg-max of the f32 per-class sums with the generated-code tie rule (running
@@ -1125,6 +1269,15 @@ hipError_t LaunchWalkRowsLds(const WalkParams &p, int interleave, int tileMode, 
   case kTileRankU8:
     if (RB != 64) return hipErrorInvalidValue;
     return LaunchWalkW<kTileRankU8>(p, interleave, prefetch, grid, block, ldsBytes, stream);
+  case kTileRankU16: // (tree groups always go straight from global memory into LDS)
+    if ((int64_t)((p.s.numFeatures + 2) / 2) * RB * 4 > 0x10000) return hipErrorInvalidValue; // byte offsets
+    switch (interleave) {
+    case 1: return LaunchWalkKP<1, 0, kTileRankU16>(p, grid, block, ldsBytes, stream);
+    case 2: return LaunchWalkKP<2, 0, kTileRankU16>(p, grid, block, ldsBytes, stream);
+    case 4: return LaunchWalkKP<4, 0, kTileRankU16>(p, grid, block, ldsBytes, stream);
+    case 8: return LaunchWalkKP<8, 0, kTileRankU16>(p, grid, block, ldsBytes, stream);
+    default: return hipErrorInvalidValue;
+    }
   default: return hipErrorInvalidValue;
   }
 }
@@ -1288,6 +1441,32 @@ hipError_t LaunchBinRows(const float *x, const float *table, uint8_t *ranks, int
   default: return hipErrorInvalidValue;
   }
 #undef TBAMD_BIN_CASE
+}
+
+hipError_t LaunchRankRows16(const float *x, const float *tables, const RankFeatureDesc *features, const RankChunkDesc *chunks,
+                            int numChunks, uint32_t maxChunkEntries, uint32_t maxChunkFeatures, uint16_t *ranks, int64_t rows,
+                            int numFeatures, int rowsPerBlock, hipStream_t stream) {
+  if (rows <= 0) return hipSuccess;
+  const uint32_t tableRegionBytes = (maxChunkEntries * (uint32_t)sizeof(float) + 15u) & ~15u;
+  const size_t ldsBytes = (size_t)tableRegionBytes + (size_t)maxChunkFeatures * kRankStride * sizeof(float);
+  if (numChunks < 1 || ldsBytes > 160 * 1024 || rowsPerBlock < 64 || rowsPerBlock % 64 != 0) return hipErrorInvalidValue;
+  const int64_t rowBlocks = (rows + rowsPerBlock - 1) / rowsPerBlock;
+  // whole row blocks (the walk copies whole tiles), in tiles of 1024 rows: smaller row blocks are ranked up to the
+  // next multiple of 1024 rows, which the rank buffer has to hold
+  const int64_t rowTiles = (rowBlocks * rowsPerBlock + kRankTileRows - 1) / kRankTileRows;
+  // enough blocks to fill the chip, each amortising its table load over a few thousand rows
+  int64_t perBlock = (rowTiles * numChunks + 4095) / 4096;
+  if (perBlock < 2) perBlock = 2;
+  if (perBlock > 16) perBlock = 16;
+  const int64_t ranges = (rowTiles + perBlock - 1) / perBlock;
+  const int64_t blocks = (ranges + 7) / 8 * 8 * numChunks; // row ranges padded to the 8 XCDs
+  if (blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
+  hipError_t e = AllowFullLds<&RankRows16Kernel>();
+  if (e != hipSuccess) return e;
+  RankRows16Kernel<<<dim3((unsigned)blocks), dim3(kRankWaves * 64), ldsBytes, stream>>>(
+      x, tables, features, chunks, reinterpret_cast<uint32_t *>(ranks), rows, numFeatures, rowsPerBlock, numChunks, (int)perBlock,
+      rowTiles, tableRegionBytes);
+  return hipGetLastError();
 }
 
 hipError_t LaunchFinalize(const FinalizeParams &p, hipStream_t stream) {

@@ -21,7 +21,7 @@ namespace tbamd {
 namespace {
 
 constexpr char kMagic[8] = {'T', 'B', 'A', 'M', 'D', 'M', 'D', 'L'};
-constexpr uint32_t kVersion = 3;
+constexpr uint32_t kVersion = 4;
 
 struct Writer {
   std::string bytes;
@@ -76,6 +76,7 @@ void SaveCompiledModel(const std::string &path, const Forest &forest, const Laun
   w.Put<int32_t>(plan.treeSlices);
   w.Put<int32_t>(plan.featureOffsetInWords ? 1 : 0);
   w.Put<int32_t>(plan.quantizedRows ? 1 : 0);
+  w.Put<int32_t>(plan.rankRows16 ? 1 : 0);
   w.Put<int32_t>(plan.tileSize);
   w.Put<int32_t>(plan.tiling);
   w.Put<int32_t>(plan.peelWalks ? 1 : 0);
@@ -120,6 +121,7 @@ CompiledModel LoadCompiledModel(const std::string &path) {
   m.plan.treeSlices = r.Get<int32_t>();
   m.plan.featureOffsetInWords = r.Get<int32_t>() != 0;
   m.plan.quantizedRows = r.Get<int32_t>() != 0;
+  m.plan.rankRows16 = r.Get<int32_t>() != 0;
   m.plan.tileSize = r.Get<int32_t>();
   m.plan.tiling = r.Get<int32_t>();
   m.plan.peelWalks = r.Get<int32_t>() != 0;

@@ -25,9 +25,10 @@ Forest NormalizeToLessThan(const Forest &forest) {
   return out;
 }
 
-uint32_t PackedModel::PadFeatureOffset() const { return (uint32_t)numFeatures * plan.FeatureStride(); }
+uint32_t PackedModel::PadFeatureOffset() const { return plan.FeatureOffset((uint32_t)numFeatures); }
 
 size_t PackedModel::RowTileBytes() const {
+  if (plan.rankRows16) return (size_t)((numFeatures + 2) / 2) * plan.rowsPerBlock * 4; // pairs of two-byte ranks, pad feature included
   return (size_t)(numFeatures + 1) * plan.rowsPerBlock * (plan.quantizedRows ? 1 : 4);
 }
 
@@ -439,11 +440,13 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCou
 
   if (plan.quantizedRows && (plan.kernel != LaunchPlan::Kernel::kRowParallelLds || plan.rowsPerBlock != 64))
     throw Error("rank-quantised rows need the row-parallel kernel with 64 rows per block");
+  if (plan.rankRows16 && (plan.kernel != LaunchPlan::Kernel::kRowParallelLds || plan.quantizedRows || plan.featureOffsetInWords))
+    throw Error("two-byte rank rows need the row-parallel kernel (and exclude one-byte ranks and word offsets)");
   const int T = plan.tileSize;
   if (T < 1 || T > kMaxTileSize)
     throw Error("tile size " + std::to_string(T) + " is not supported: the device kernels walk tiles of 1 to " +
                 std::to_string(kMaxTileSize) + " nodes");
-  if (T > 1 && (plan.kernel != LaunchPlan::Kernel::kRowParallelLds || plan.quantizedRows))
+  if (T > 1 && (plan.kernel != LaunchPlan::Kernel::kRowParallelLds || plan.quantizedRows || plan.rankRows16))
     throw Error("tile sizes above 1 need the row-parallel kernel on float32 rows");
   if (T > 1 && (plan.featureOffsetInWords || (int64_t)(forest.numFeatures + 1) * plan.rowsPerBlock * 4 > 0x10000))
     throw Error("tile sizes above 1 need a row tile below 64 KB (tiles hold byte offsets): fewer rows per block");
@@ -457,6 +460,7 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCou
   if (padOffset > 0xFFFFu)
     throw Error("feature offsets do not fit 16 bits for this rowsPerBlock / feature count");
   const uint32_t featureStride = plan.FeatureStride();
+  if (plan.rankRows16 && pm.RowTileBytes() > 0x10000u) throw Error("two-byte rank rows: the row tile must stay below 64 KB (byte offsets)");
   const uint32_t groupCapacity = (uint32_t)plan.groupBytes / kNodeBytes; // in 8-byte units
   const uint32_t tileUnits = TileBytes(T) / kNodeBytes;                    // units per tile (1 for scalar nodes)
 
@@ -479,6 +483,55 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCou
     for (int32_t f = 0; f < forest.numFeatures; ++f)
       for (size_t k = 0; k < ranks[f].size(); ++k)
         pm.binThresholds[((size_t)(f / chunk) * depth + k) * chunk + (f % chunk)] = ranks[f][k];
+  }
+
+  if (plan.rankRows16) {
+    ranks = ThresholdsPerFeature(forest);
+    // LDS of one block of the ranking kernel: the chunk's tables and a staging tile of 1025 floats per feature of
+    // the chunk (two blocks per compute unit)
+    constexpr size_t kChunkBytes = 76 * 1024, kStageBytesPerFeature = 1025 * 4;
+    pm.rankFeatures.resize((size_t)((forest.numFeatures + 2) / 2) * 2); // every slot of the tile, the pad feature's included
+    auto tableEntries = [&](size_t f) -> size_t {
+      if (f >= ranks.size() || ranks[f].empty()) return 0;
+      size_t entries = 1;
+      while (entries < ranks[f].size()) entries = entries * 2 + 1; // 2^n - 1 >= thresholds
+      return entries;
+    };
+    for (size_t f = 0; f < ranks.size(); ++f)
+      if (ranks[f].size() > 65534) throw Error("a feature has more than 65534 distinct thresholds: rows cannot be ranked in two bytes");
+    size_t f = 0;
+    while (f < pm.rankFeatures.size()) {
+      RankChunkDesc chunk{(uint32_t)f, 0, (uint32_t)pm.rankTables.size(), 0};
+      size_t entries = 0;
+      while (f < pm.rankFeatures.size()) {
+        const size_t pairEntries = tableEntries(f) + tableEntries(f + 1);
+        if (pairEntries * 4 + 2 * kStageBytesPerFeature > 150 * 1024) throw Error("the thresholds of one feature pair do not fit the ranking kernel's LDS");
+        if (chunk.numFeatures > 0 && (entries + pairEntries) * 4 + (chunk.numFeatures + 2) * kStageBytesPerFeature > kChunkBytes) break;
+        for (size_t g = f; g < f + 2; ++g) {
+          const size_t n = tableEntries(g);
+          uint32_t levels = 0;
+          while (((size_t)1 << levels) - 1 < n) ++levels;
+          pm.rankFeatures[g] = RankFeatureDesc{(uint32_t)entries, levels};
+          // breadth-first order of the complete search tree over the sorted thresholds (+inf beyond the last)
+          std::vector<float> bfs(n, std::numeric_limits<float>::infinity());
+          std::function<void(size_t, size_t, size_t)> fill = [&](size_t node, size_t lo, size_t hi) { // keys [lo, hi)
+            if (node >= n) return;
+            const size_t mid = lo + (hi - lo) / 2;
+            if (mid < ranks[g].size()) bfs[node] = ranks[g][mid];
+            fill(2 * node + 1, lo, mid);
+            fill(2 * node + 2, mid + 1, hi);
+          };
+          fill(0, 0, n);
+          pm.rankTables.insert(pm.rankTables.end(), bfs.begin(), bfs.end());
+          entries += n;
+        }
+        chunk.numFeatures += 2;
+        f += 2;
+      }
+      chunk.tableEntries = (uint32_t)entries;
+      pm.rankChunks.push_back(chunk);
+    }
+    pm.rankThresholds = ranks;
   }
 
   // Per tree: its size in the packed layout, the steps of a lock-step walk, and the steps after which the walk
@@ -604,7 +657,7 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCou
       const int32_t n = lo.order[i];
       DeviceNode dn;
       dn.value = tree.value[n];
-      if (plan.quantizedRows && !tree.IsLeaf(n)) {
+      if ((plan.quantizedRows || plan.rankRows16) && !tree.IsLeaf(n)) {
         const auto &sorted = ranks[(size_t)tree.feature[n]];
         const uint32_t j = (uint32_t)(std::lower_bound(sorted.begin(), sorted.end(), tree.value[n]) - sorted.begin());
         static_assert(sizeof(float) == sizeof(uint32_t), "node value holds the rank bit pattern");
@@ -616,7 +669,7 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCou
         const uint32_t child = base + (uint32_t)lo.position[tree.left[n]];
         if (lo.position[tree.right[n]] != lo.position[tree.left[n]] + 1)
           throw Error("internal error: siblings not adjacent");
-        dn.meta = ((child * kNodeBytes) << 16) | ((uint32_t)tree.feature[n] * featureStride);
+        dn.meta = ((child * kNodeBytes) << 16) | plan.FeatureOffset((uint32_t)tree.feature[n]);
       }
       pm.nodes.push_back(dn);
       pm.nodeOrigin.push_back(n);
@@ -758,8 +811,13 @@ Tree UnpackTree(const PackedModel &pm, int32_t treeIndex) {
             const int32_t chunk = pm.binChunkFeatures;
             tree.value[me] = pm.binThresholds[((size_t)(f / chunk) * pm.binTableDepth + j) * chunk + (f % chunk)];
           }
+          if (child != q && pm.plan.rankRows16) {
+            uint32_t j;
+            std::memcpy(&j, &dn.value, sizeof(j));
+            tree.value[me] = pm.rankThresholds.at(pm.plan.FeatureOfOffset(dn.meta & 0xFFFFu)).at(j);
+          }
           if (child != q) {
-            tree.feature[me] = (int32_t)((dn.meta & 0xFFFFu) / featureStride);
+            tree.feature[me] = (int32_t)pm.plan.FeatureOfOffset(dn.meta & 0xFFFFu);
             tree.left[me] = pm.nodeOrigin[g.nodeBegin + child];
             tree.right[me] = pm.nodeOrigin[g.nodeBegin + child + 1];
           }

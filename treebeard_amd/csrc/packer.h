@@ -33,6 +33,10 @@ struct LaunchPlan {
   // by the number of that feature's split thresholds that are <= it (one byte), which preserves the
   // outcome of every comparison; 64 rows of 1 byte per feature then fit LDS where 64 f32 rows do not.
   bool quantizedRows = false;
+  // The same idea for narrow models whose features have up to 65534 distinct thresholds: two-byte ranks, made by
+  // a separate kernel and laid out as [row block][feature pair][row][2], so that a row's LDS column keeps one bank
+  // of its own and the tile takes half the bytes of f32 rows (more rows per block, bigger tree groups).
+  bool rankRows16 = false;
   // Tiled walk (row-parallel kernel on f32 rows only): nodes per tile (up to 8), 1 = scalar nodes.  How the members of a
   // tile are chosen follows the reference: 0 breadth first (src/mlir/UniformTilingTransformation.cpp:148-195),
   // 1 most-visited child first on trees whose profile is skewed, 2 the same but breadth first below nodes that
@@ -54,6 +58,15 @@ struct LaunchPlan {
     if (kernel == Kernel::kTreeParallel) return 4u;
     if (quantizedRows) return (uint32_t)rowsPerBlock / 4u; // byte tile, offsets in units of 4 bytes
     return featureOffsetInWords ? (uint32_t)rowsPerBlock : (uint32_t)rowsPerBlock * 4u;
+  }
+  // What a node stores for feature f (f = numFeatures: the pad feature).
+  uint32_t FeatureOffset(uint32_t f) const {
+    if (rankRows16) return (f >> 1) * (uint32_t)rowsPerBlock * 4u + (f & 1u) * 2u; // byte offset in the [pair][row][2] tile
+    return f * FeatureStride();
+  }
+  uint32_t FeatureOfOffset(uint32_t offset) const {
+    if (rankRows16) return offset / ((uint32_t)rowsPerBlock * 4u) * 2u + ((offset >> 1) & 1u);
+    return offset / FeatureStride();
   }
 };
 
@@ -87,6 +100,15 @@ struct PackedModel {
   std::vector<float> binThresholds;
   int32_t binTableDepth = 0;
   int32_t binChunkFeatures = 0;
+  // Two-byte ranks (plan.rankRows16): the thresholds of every feature as a complete search tree in breadth-first
+  // order (root, its two children, ...; 2^levels - 1 entries, +inf behind the feature's last threshold), feature
+  // after feature; the ranking kernel's blocks each take one chunk of whole feature pairs whose tables fit LDS.
+  // RankFeatureDesc: the feature's first table entry relative to its chunk's first entry, and its search steps
+  // (0: no threshold); RankChunkDesc: whole pairs (firstFeature is even) and the chunk's tables in rankTables.
+  std::vector<float> rankTables;
+  std::vector<std::vector<float>> rankThresholds; // per feature, sorted (host side only: unpacking and checks)
+  std::vector<RankFeatureDesc> rankFeatures;      // one per slot of the tile: (numFeatures + 2) / 2 pairs
+  std::vector<RankChunkDesc> rankChunks;
 
   uint32_t PadFeatureOffset() const;
   // LDS bytes of the tree-group region (regressors reuse it for the tree threads' cross-wave pass).

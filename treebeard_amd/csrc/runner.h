@@ -159,7 +159,10 @@ private:
   int32_t *m_dSlotTree = nullptr;
   double *m_dPartial = nullptr;
   size_t m_partialBytes = 0;
-  float *m_dBinTable = nullptr;
+  float *m_dBinTable = nullptr;                 // threshold tables of the rank-quantising kernels (one- or two-byte ranks)
+  RankFeatureDesc *m_dRankFeatures = nullptr;   // two-byte ranks: per-feature table index
+  RankChunkDesc *m_dRankChunks = nullptr;
+  uint32_t m_rankChunkEntries = 0, m_rankChunkFeatures = 0; // the largest chunk: the ranking kernel's LDS need
   uint8_t *m_dRanks = nullptr;
   size_t m_ranksBytes = 0;
   float *m_dStageIn = nullptr;

@@ -374,6 +374,7 @@ int32_t tbmi_set_plan(intptr_t h, int32_t rowsPerBlock, int32_t treeThreads, int
         plan.kernel = LaunchPlan::Kernel::kRowParallelLds;
         plan.treeLanes = 1;
         plan.quantizedRows = false;
+        plan.rankRows16 = false;
         if (rowsPerBlock > 0) plan.rowsPerBlock = rowsPerBlock;
         plan.treeThreads = treeThreads > 0 ? treeThreads : 1;
         if (interleave > 0) plan.interleave = interleave;
@@ -396,6 +397,7 @@ int32_t tbmi_set_tree_parallel_plan(intptr_t h, int32_t rowsPerBlock, int32_t tr
         plan.kernel = LaunchPlan::Kernel::kTreeParallel;
         plan.featureOffsetInWords = false;
         plan.quantizedRows = false;
+        plan.rankRows16 = false;
         plan.treeThreads = 1;
         plan.rowsPerBlock = rowsPerBlock;
         plan.treeLanes = treeLanes;
@@ -438,10 +440,34 @@ int32_t tbmi_set_quantized_plan(intptr_t h, int32_t treeThreads, int32_t interle
         LaunchPlan plan = r->Model().plan;
         plan.kernel = LaunchPlan::Kernel::kRowParallelLds;
         plan.quantizedRows = true;
+        plan.rankRows16 = false;
         plan.featureOffsetInWords = false;
         plan.rowsPerBlock = 64;
         plan.treeLanes = 1;
         plan.treeThreads = treeThreads > 0 ? treeThreads : 8;
+        plan.interleave = interleave > 0 ? interleave : 4;
+        if (groupBytes > 0) plan.groupBytes = groupBytes;
+        else plan.groupBytes = std::min(plan.groupBytes, 256 * plan.ThreadsPerBlock());
+        plan.treeSlices = treeSlices > 0 ? treeSlices : 1;
+        r->Repack(plan);
+        return 0;
+      },
+      -1);
+}
+
+int32_t tbmi_set_rank16_plan(intptr_t h, int32_t rowsPerBlock, int32_t treeThreads, int32_t interleave, int32_t groupBytes,
+                             int32_t treeSlices) {
+  return Guard(
+      [&] {
+        InferenceRunner *r = Runner(h);
+        LaunchPlan plan = r->Model().plan;
+        plan.kernel = LaunchPlan::Kernel::kRowParallelLds;
+        plan.rankRows16 = true;
+        plan.quantizedRows = false;
+        plan.featureOffsetInWords = false;
+        plan.treeLanes = 1;
+        plan.rowsPerBlock = rowsPerBlock > 0 ? rowsPerBlock : 256;
+        plan.treeThreads = treeThreads > 0 ? treeThreads : std::max(1, 1024 / plan.rowsPerBlock);
         plan.interleave = interleave > 0 ? interleave : 4;
         if (groupBytes > 0) plan.groupBytes = groupBytes;
         else plan.groupBytes = std::min(plan.groupBytes, 256 * plan.ThreadsPerBlock());

@@ -346,6 +346,23 @@ std::vector<LaunchPlan> CandidatePlans(const Forest &forest, int64_t batchSize, 
                           q.interleave == p.interleave && q.groupBytes == p.groupBytes);
           if (!dup) out.push_back(p);
         }
+  // Two-byte rank rows (a ranking kernel in front of the walk, half the row tile): the timed search counts both
+  // kernels, so the form is kept only where the walk gains more than the ranking costs.
+  if (!base.quantizedRows && base.treeSlices == 1)
+    for (int32_t rb : {256, 512}) {
+      const int64_t rowTile = (int64_t)((forest.numFeatures + 2) / 2) * rb * 4;
+      if (rowTile > 0xFFFF) continue;
+      LaunchPlan p = base;
+      p.rankRows16 = true;
+      p.featureOffsetInWords = false;
+      p.rowsPerBlock = rb;
+      p.treeThreads = 1024 / rb;
+      p.interleave = 4;
+      int64_t group = std::min<int64_t>(65536, limits.ldsBytesPerBlock / 2 - rowTile - (forest.numClasses > 0 ? 1024 * 8 : 0) - 2048);
+      if (group < need || group < 8192) continue;
+      p.groupBytes = (int32_t)(group & ~15);
+      out.push_back(p);
+    }
   return out;
 }
 

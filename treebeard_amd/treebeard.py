@@ -352,6 +352,10 @@ class TreebeardInferenceRunner:
         """0 by rule, 1 tree groups through prefetch registers, 2 direct global-to-LDS copies."""
         self._rc(_lib().tbmi_set_group_staging(self.inferenceRunner, mode), "tbmi_set_group_staging")
 
+    def set_rank16_plan(self, rows_per_block=256, tree_threads=0, interleave=4, group_bytes=0, tree_slices=1):
+        self._rc(_lib().tbmi_set_rank16_plan(self.inferenceRunner, rows_per_block, tree_threads, interleave, group_bytes,
+                                             tree_slices), "tbmi_set_rank16_plan")
+
     def set_quantized_plan(self, tree_threads=8, interleave=4, group_bytes=0, tree_slices=1):
         self._rc(_lib().tbmi_set_quantized_plan(self.inferenceRunner, tree_threads, interleave, group_bytes,
                                                 tree_slices), "tbmi_set_quantized_plan")
