@@ -179,12 +179,46 @@ void WalkRowLds(const WalkParams &p, int K, uint32_t stride, int rankRows, int64
             const uint32_t rank = (int)f == F ? 0u : ranks[((row / 64) * F + f) * 64 + (row % 64)];
             left = rank <= Bits(node.value);
           } else {
-            const float x = (int)f == F ? -INFINITY : p.x[row * F + f];
+            const float x = (int)f >= F ? -INFINITY : p.x[row * F + f]; // (the pad feature and the stub feature hold -inf)
             left = x < node.value;
           }
           addr = (node.meta >> 16) + (left ? 0u : kNodeBytes);
         }
         if (addr / kNodeBytes >= grp.nodeCount) std::abort();
+        bool inTail = false;
+        uint32_t at = 0;
+        if (p.s.deferTails) {
+          // a stub (NaN value, child pointer one node before itself) stands for the node of the tail array its
+          // payload names: the walk goes on there for at most tailDepth steps
+          const DeviceNode stop = nodes[grp.nodeBegin + addr / kNodeBytes];
+          if (rankRows != 0 || stride == 0) std::abort();
+          if (stop.value != stop.value) { // a NaN marks a stub; its payload is the tail index
+            if (!bd.hasStubs || (stop.meta >> 16) + kNodeBytes != addr || (Bits(stop.value) & ~kStubIndexMask) != kStubValueBits ||
+                !p.tailNodes || !p.tailOrigin)
+              std::abort();
+            inTail = true;
+            at = Bits(stop.value) & kStubIndexMask;
+            if (at == 0) std::abort();
+            for (int d = 0; d < p.s.tailDepth; ++d) {
+              const DeviceNode node = p.tailNodes[at];
+              const uint32_t f = node.meta & ((1u << kTailFeatureBits) - 1u);
+              if ((int)f > F) std::abort();
+              const float x = (int)f == F ? -INFINITY : p.x[row * F + f];
+              at = (node.meta >> kTailFeatureBits) + (x < node.value ? 0u : 1u);
+            }
+            const DeviceNode leaf = p.tailNodes[at];
+            if ((leaf.meta >> kTailFeatureBits) != at || (leaf.meta & ((1u << kTailFeatureBits) - 1u)) != (uint32_t)F) std::abort(); // tailDepth must reach a leaf
+          }
+        }
+        if (inTail) {
+          classSums[0] += (double)p.tailNodes[at].value;
+          classSeen[0] = true;
+          if (p.leafIds) {
+            const int tree = p.slotTree[bd.firstSlot + k];
+            if (tree >= 0) p.leafIds[row * p.s.numTrees + tree] = p.tailOrigin[at];
+          }
+          continue;
+        }
         const int cls = p.s.numClasses > 0 ? (int)bd.classId : 0;
         classSums[cls] += (double)nodes[grp.nodeBegin + addr / kNodeBytes].value;
         classSeen[cls] = true;

@@ -1055,16 +1055,13 @@ def test_profiled_runner_selects_the_same_leaves(synth_model, plain_file, tmp_pa
 
 
 def test_describe_plan_says_where_walk_peeling_applies(synth_model, tmp_path):
-    """Peeled walks exist for the tiled kernel and for the scalar row-parallel kernel that stores sums; a
-    classifier whose walk kernel keeps the arg-max itself walks every bundle to its full depth, and says so."""
+    """Peeled walks exist for the tiled kernel and, as deferred tails, for the scalar row-parallel kernel on models
+    without classes; elsewhere every bundle walks its full depth, and the plan description says so."""
     forest = model_io.load_xgboost_json(synth_model(3))
     x = synth.CONFIGS[3].batch_rows(1000, seed_offset=3)
     profile = write_profile(tmp_path / "c3.profile.csv", forest, cpu_oracle.leaf_ids(forest, synth.CONFIGS[3].batch_rows(2000)))
-    runner = make_tiled_runner(synth_model(3), 1 << 17, 1, 1, profile, True, multiclass=True)   # (a batch that needs one tree slice)
-    assert " treeSlices=1 " in runner.describe_plan() and " peelWalks=ignored(fused) " in runner.describe_plan()
-    check_against_oracle(runner, forest, x)
-    runner.set_plan(128, 8, 4, 0, 2)                  # two tree slices: sums go through the finalize kernel
-    assert " peelWalks=1 " in runner.describe_plan()
+    runner = make_tiled_runner(synth_model(3), 1 << 17, 1, 1, profile, True, multiclass=True)
+    assert " peelWalks=ignored(classes) " in runner.describe_plan()
     check_against_oracle(runner, forest, x)
     runner.set_tree_parallel_plan(4, 64, 1, 0, 1)
     assert " peelWalks=ignored(tree_parallel) " in runner.describe_plan()
@@ -1073,6 +1070,73 @@ def test_describe_plan_says_where_walk_peeling_applies(synth_model, tmp_path):
     check_against_oracle(tiled, forest, x)
     with pytest.raises(RuntimeError, match="row-parallel"):
         tiled.set_global_walk_plan(256, 4, 1)         # a tiled runner does not quietly become a scalar walk
+    forest5 = model_io.load_xgboost_json(synth_model(5))
+    profile5 = write_profile(tmp_path / "c5.profile.csv", forest5, cpu_oracle.leaf_ids(forest5, synth.CONFIGS[5].batch_rows(2000)))
+    scalar = make_tiled_runner(synth_model(5), 4000, 1, 1, profile5, True)
+    assert " peelWalks=1 " in scalar.describe_plan() and int(scalar.describe_plan().split("treesDeferred=")[1].split()[0]) > 100
+    scalar.set_rank16_plan(128, 8, 4, 0, 1)
+    assert " peelWalks=ignored(ranks) " in scalar.describe_plan()
+
+
+@pytest.mark.parametrize("plan", [None, (256, 4, 4, 0, 1), (128, 8, 2, 24576, 3), (64, 4, 8, 16384, 7), (512, 2, 1, 32768, 1), (64, 16, 4, 0, 1)])
+@pytest.mark.parametrize("k", [2, 5])
+def test_deferred_tails_select_the_same_leaves(synth_model, tmp_path, k, plan):
+    """Peeled walks of the scalar kernel: trees whose walks stop at a profiled level, the rows that stand on a stub
+    queued per wave and walked on densely through the tail array in global memory.  Leaf ids bit-exact and the
+    predictions those of an unprofiled runner, for several block shapes and tree slices, with the profile taken
+    from other rows than the batch, +-inf and NaN rows, a batch that ends inside a row block, every entry point."""
+    forest = model_io.load_xgboost_json(synth_model(k))
+    rows = 5000 + 37
+    x = synth.CONFIGS[k].batch_rows(rows, seed_offset=8)
+    x[3, :] = np.inf
+    x[4, :] = -np.inf
+    x[5, ::3] = np.nan
+    profile = write_profile(tmp_path / "profile.csv", forest, cpu_oracle.leaf_ids(forest, synth.CONFIGS[k].batch_rows(3000)))
+    plain = make_tiled_runner(synth_model(k), rows, 1)
+    runner = make_tiled_runner(synth_model(k), rows, 1, 1, profile, True)
+    if plan and plan[0] * (forest.num_features + 1) * 4 > 150 * 1024:
+        with pytest.raises(RuntimeError, match="exceeds the LDS"):
+            runner.set_plan(*plan)
+        return
+    if plan:
+        runner.set_plan(*plan)
+    described = runner.describe_plan()
+    if " peelWalks=1 " in described:
+        assert int(described.split("treesDeferred=")[1].split()[0]) > 100, described
+    else:       # a shape without room for the form says so and walks every tree to its leaves (wide row tiles, small tree groups)
+        assert plan and (" peelWalks=ignored(words) " in described or " peelWalks=ignored(lds) " in described), described
+    check_against_oracle(runner, forest, x)
+    expected = gpu_predict(plain, x)
+    np.testing.assert_allclose(gpu_predict(runner, x), expected, rtol=1e-6, atol=1e-7)    # (the tails' leaf values join the sum in another order)
+    np.testing.assert_allclose(runner.RunInference(x), expected, rtol=1e-6, atol=1e-7)
+    dx = torch.from_numpy(x).cuda()
+    got = torch.zeros(rows, dtype=torch.float32, device="cuda")
+    stream = torch.cuda.current_stream()
+    runner.run_device_noalloc(dx.data_ptr(), got.data_ptr(), rows, stream.cuda_stream)
+    stream.synchronize()
+    np.testing.assert_allclose(got.cpu().numpy(), expected, rtol=1e-6, atol=1e-7)
+    small = gpu_predict(runner, x[:70])                  # a batch of two row blocks at most: everything leaves through the last flush
+    np.testing.assert_allclose(small, expected[:70], rtol=1e-6, atol=1e-7)
+
+
+def test_deferred_tails_survive_the_compiled_model_file_and_the_plan_search(synth_model, tmp_path):
+    forest = model_io.load_xgboost_json(synth_model(5))
+    rows = 1 << 15
+    x = synth.CONFIGS[5].batch_rows(rows, seed_offset=9)
+    profile = write_profile(tmp_path / "profile.csv", forest, cpu_oracle.leaf_ids(forest, x[:3000]))
+    runner = make_tiled_runner(synth_model(5), rows, 1, 1, profile, True)
+    path = str(tmp_path / "deferred.tbamd")
+    runner.save_compiled_model(path)
+    again = treebeard.TreebeardInferenceRunner.FromSOFile(path, "")
+    assert again.describe_plan() == runner.describe_plan() and " peelWalks=1 " in again.describe_plan()
+    check_against_oracle(again, forest, x[:4096])
+    # the plan search of a runner without a profile profiles the batch itself and may keep deferred tails; whatever
+    # it keeps selects the same leaves
+    tuned = make_runner(synth_model(5), rows)
+    dx = torch.from_numpy(x).cuda()
+    torch.cuda.synchronize()
+    tuned.autotune(dx.data_ptr(), rows)
+    check_against_oracle(tuned, forest, x[:4096])
 
 
 @pytest.mark.parametrize("features,rows", [(20000, 300), (40000, 70)])

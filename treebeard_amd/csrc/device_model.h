@@ -19,6 +19,15 @@
 //    whose column holds -inf: `x < value` is then always true, the walk takes
 //    the "left" pointer and stays on the leaf.  A walk of `depth` steps thus
 //    needs no leaf test: it ends on the leaf for every row.
+//  * Deferred tails (LaunchPlan::deferTails; the reference's peeled walks for skewed trees,
+//    src/mlir/ProbabilityBasedTilingTransform.cpp:66-73, src/mlir/WalkDecisionTreeLoweringPass.cpp:231-315): the
+//    lock-step walk of a tree may stop at a level above its leaves.  The internal nodes of that level are then
+//    represented by STUBS, which hold the walk in place like a leaf: the value field is a NaN (every compare
+//    fails, the walk takes the "right" child) and the child pointer is the stub's own address minus one node, so
+//    the right child is the stub itself.  The NaN's payload is the index of the node the stub stands for in the
+//    TAIL ARRAY: the subtrees below the stubs stay in global memory, out of the tree groups, as nodes
+//    { value; (left child index << kTailFeatureBits) | feature index } (PackedModel::tailNodes).  A model with a
+//    NaN leaf value keeps its trees whole.
 //  * Trees are walked K at a time (a BUNDLE) to give every lane K independent
 //    dependency chains.  A bundle records the K root addresses, the trip count
 //    (deepest tree of the bundle) and the class the trees add to.
@@ -59,6 +68,14 @@ namespace tbamd {
 
 constexpr int kMaxInterleave = 8;
 constexpr uint32_t kNodeBytes = 8;
+constexpr uint32_t kDeferBytesPerWave = 512; // LDS of one wave's queue of deferred walks (LaunchPlan::deferTails)
+// Deferred tails: a tail node's meta word holds the index of its left child above kTailFeatureBits bits of feature
+// index; a queue entry holds a tail index below 6 bits of lane (bits 26 to 31).
+constexpr uint32_t kTailFeatureBits = 12;
+constexpr uint32_t kMaxTailNodes = 1u << 20;
+// A stub's value field: a quiet NaN whose low bits are the tail index.
+constexpr uint32_t kStubValueBits = 0x7FC00000u;
+constexpr uint32_t kStubIndexMask = kMaxTailNodes - 1u;
 constexpr int kMaxTileSize = 8;
 // Tiles of more than kMaxSelectTile nodes carry links instead of a child-select table.
 constexpr int kMaxSelectTile = 4;
@@ -79,8 +96,9 @@ struct DeviceNode {
 
 struct alignas(32) DeviceBundle {
   uint16_t root[kMaxInterleave]; // byte address of each tree's root inside the group
-  uint32_t depth;                // walk steps (tile steps in the tiled layout) that bring every row to a leaf
-  uint32_t classId;              // (32-bit fields: the kernels fetch a bundle with scalar loads only)
+  uint32_t depth;                // walk steps (tile steps in the tiled layout) that bring every row to a leaf (or to a stub)
+  uint16_t classId;              // (the kernels fetch a bundle with scalar loads only)
+  uint16_t hasStubs;             // deferred tails: some tree of the bundle ends in stubs
   uint32_t firstSlot;            // index of root[0] in the slot->tree table
   uint32_t peelDepth;            // steps taken without looking; the rest runs while any lane still moves (== depth: no tail)
 };

@@ -23,6 +23,10 @@ struct WalkScalars {
   // Row-parallel kernels, classifiers with one tree slice: the kernel keeps the running arg-max of the class
   // sums (which arrive in ascending class order) and stores the class id itself; no partial sums, no finalize.
   int32_t fuseArgmax = 0;
+  // Scalar row-parallel walk on an f32 tile with byte offsets: trees may end in stubs (device_model.h); the row
+  // tile then has a column for the stub feature and every wave a queue of deferred walks behind it.
+  int32_t deferTails = 0;
+  int32_t tailDepth = 0;         // steps the deepest deferred walk takes below its stub
   double initialValue = 0.0;
 };
 
@@ -33,9 +37,11 @@ struct WalkParams {
   const DeviceBundle *bundles = nullptr;
   const DeviceNode *bundleRoots = nullptr; // interleave root-node copies per bundle (row-parallel f32 walk)
   const DeviceGroup *groups = nullptr;
+  const DeviceNode *tailNodes = nullptr;   // deferred tails: the subtrees below the stubs (PackedModel::tailNodes)
+  const int32_t *tailOrigin = nullptr;     // ... and their original node ids (leaf-id dump)
   const DeviceGlobalNode *globalNodes = nullptr; // global-memory walk only
   const DeviceGlobalTree *globalTrees = nullptr;
-  bool peelWalks = false;         // bundles carry peel depths below their depths: use the kernels that look at them
+  bool peelWalks = false;         // tiled walk: bundles carry peel depths below their depths
   // Row-parallel scalar walk: tree groups go straight from global memory into LDS (no staging registers); the
   // block waits for its copy, so this pays when a second block on the CU walks meanwhile.
   bool directStaging = false;

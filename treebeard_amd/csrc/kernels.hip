@@ -124,15 +124,21 @@ __device__ __forceinline__ void StageRows(const float *__restrict__ src, int val
 // without growing the row tile; their sums meet in an LDS cross-wave pass.
 // Sums are kept in double; trees are added in packed order.
 // ---------------------------------------------------------------------------
-// kPeel: bundles carry a peel depth taken from a hit-count profile (the steps that bring 90 % of the profiled
-// rows to a leaf, src/mlir/ProbabilityBasedTilingTransform.cpp:66-73): the walk takes that many steps blind and
-// then goes on only while some lane of the wave still moves, at most to the full depth.  Without kPeel the
-// peel depth is not looked at and every bundle walks its full depth.
+// kDefer (peeled walks, src/mlir/ProbabilityBasedTilingTransform.cpp:66-73, src/mlir/WalkDecisionTreeLoweringPass.cpp
+// :231-315, the way this hardware wants them): the lock-step walk of a tree stops at the level a hit-count
+// profile says it still pays (device_model.h: stubs).  A row that ends on a stub is queued by its wave as
+// (row, tail node); whenever 64 entries have come together - whatever trees they belong to - the wave walks
+// them on densely, one entry per lane, to their leaves, and hands the leaf values back to the rows' lanes
+// through LDS.  The subtrees below the stubs are not part of the tree groups: the dense walk reads its nodes
+// from global memory (they stay in L2), so the queue outlives the groups and is emptied once more at the end.
+// Lock step spends its LDS reads on all 64 rows of a wave even when three of them still move; the queue spends
+// 64 lanes on 64 rows that do, its node reads go through the vector memory path, which the walk leaves idle,
+// and only its feature reads (at scattered addresses now) come out of LDS.
 //
 // kVariant picks what is compiled in beside the plain walk (each costs the plain walk about a percent when it
-// is merely present): kWalkDump the leaf-id dump of the parity checks, kWalkPeel the peeled walk, kWalkFuse the
-// classifiers' running arg-max (WalkScalars::fuseArgmax).
-enum WalkVariant : int { kWalkPlain = 0, kWalkDump = 1, kWalkPeel = 2, kWalkFuse = 3 };
+// is merely present): kWalkDump the leaf-id dump of the parity checks, kWalkDefer the deferred tails, kWalkFuse
+// the classifiers' running arg-max (WalkScalars::fuseArgmax).
+enum WalkVariant : int { kWalkPlain = 0, kWalkDump = 1, kWalkDefer = 2, kWalkFuse = 3 };
 
 template <int K, int PF, int kMode, int kVariant>
 __global__ void __launch_bounds__(1024)
@@ -141,8 +147,8 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
                   const DeviceGroup *__restrict__ groups,
                   const WalkScalars s, float *__restrict__ out, int8_t *__restrict__ classOut,
                   double *__restrict__ partial, int32_t *__restrict__ leafIds, const int32_t *__restrict__ nodeOrigin,
-                  const int32_t *__restrict__ slotTree) {
-  constexpr bool kDump = kVariant == kWalkDump, kPeel = kVariant == kWalkPeel, kFuse = kVariant == kWalkFuse;
+                  const int32_t *__restrict__ slotTree, const U32x2 *__restrict__ tailNodes, const int32_t *__restrict__ tailOrigin) {
+  constexpr bool kDump = kVariant == kWalkDump, kDefer = kVariant == kWalkDefer, kFuse = kVariant == kWalkFuse;
   // LDS: [tree group nodes | transposed row tile].  The group sits at LDS
   // address 0 so that node pointers are LDS addresses as stored.
   extern __shared__ __align__(16) unsigned char lds[];
@@ -193,6 +199,15 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
     for (int i = tid; i < RB; i += threads) rowTile[F * RB + i] = -INFINITY; // pad feature: keeps leaves in place
     column = s.groupRegionBytes + (uint32_t)lane * 4u;
   }
+  // Deferred tails: the wave's queue of (row, node) entries, 128 of 4 bytes behind the row tile; while the wave
+  // walks 64 of them on, the same 512 bytes take the leaf values on their way back (a double per lane).
+  const uint32_t queueAddress = ((s.groupRegionBytes + (uint32_t)(F + 1) * RB * 4u + 15u) & ~15u) +
+                                (uint32_t)__builtin_amdgcn_readfirstlane(tid >> 6) * kDeferBytesPerWave;
+  uint32_t *queue = reinterpret_cast<uint32_t *>(lds + queueAddress);
+  double *handBack = reinterpret_cast<double *>(lds + queueAddress);
+  const uint32_t waveColumn = column - (uint32_t)(tid & 63) * 4u; // LDS address of feature 0 of the wave's first row
+  const uint32_t laneTag = (uint32_t)(tid & 63) << 26;            // a queue entry: lane << 26 | tail index
+  uint32_t queued = 0;                                            // entries in the queue (the same in every lane)
 
   const int slice = blockIdx.y;
   const int gBegin = (int)(((int64_t)s.numGroups * slice) / s.treeSlices);
@@ -253,6 +268,48 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
       for (int c = curClass + 1; c < (UPTO); ++c) partialRow[c] = 0.0;                                                 \
     }                                                                                                                  \
     acc = 0.0;                                                                                                         \
+  }
+  // Walks the first 64 (or fewer) entries of the wave's queue to their leaves, one entry per lane, and adds the
+  // leaf values to the sums of the rows they belong to; what the queue holds beyond 64 moves to its front.  A
+  // lane without an entry walks tail node 0, a leaf of value 0.  Only LDS accesses of this one wave touch the
+  // queue, and a wave's LDS accesses complete in program order.
+  const uint32_t tileShift = (uint32_t)__builtin_ctz((unsigned)RB) + 2u; // feature index -> byte offset in the row tile
+#define TBAMD_WALK_QUEUE                                                                                               \
+  {                                                                                                                    \
+    const uint32_t me = (uint32_t)(tid & 63);                                                                          \
+    const uint32_t take = queued < 64u ? queued : 64u;                                                                 \
+    const uint32_t entry = me < take ? queue[me] : 0u;                                                                 \
+    const uint32_t later = 64u + me < queued ? queue[64u + me] : 0u;                                                   \
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                                             \
+    __builtin_amdgcn_wave_barrier();                                                                                   \
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");                                                             \
+    handBack[me] = 0.0;                                                                                                \
+    uint32_t at = entry & kStubIndexMask;                                                                              \
+    const uint32_t owner = entry >> 26;                                                                                \
+    const uint32_t ownerColumn = waveColumn + owner * 4u;                                                              \
+    U32x2 node = tailNodes[at];                                                                                        \
+    for (int d = 0; d < s.tailDepth; ++d) {                                                                            \
+      const bool left = LdsLoadFloat(ownerColumn + ((node.y & ((1u << kTailFeatureBits) - 1u)) << tileShift)) < AsFloat(node.x); \
+      const uint32_t next = (node.y >> kTailFeatureBits) + (left ? 0u : 1u);                                           \
+      const bool moved = next != at;                                                                                   \
+      at = next;                                                                                                       \
+      if (!__any(moved)) break;                                                                                        \
+      node = tailNodes[at];                                                                                            \
+    }                                                                                                                  \
+    const double leafValue = (double)AsFloat(node.x);                                                                  \
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                                             \
+    __builtin_amdgcn_wave_barrier();                                                                                   \
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");                                                             \
+    if (me < take) __hip_atomic_fetch_add(&handBack[owner], leafValue, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT); \
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                                             \
+    __builtin_amdgcn_wave_barrier();                                                                                   \
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");                                                             \
+    acc += handBack[me];                                                                                               \
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                                             \
+    __builtin_amdgcn_wave_barrier();                                                                                   \
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");                                                             \
+    if (64u + me < queued) queue[me] = later;                                                                          \
+    queued = queued > 64u ? queued - 64u : 0u;                                                                         \
   }
   if (PF > 0 && gBegin < gEnd) TBAMD_PREFETCH_GROUP(groups[gBegin])
 
@@ -324,9 +381,8 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
             addr[k] = (root.meta >> 16) + (left ? 0u : kNodeBytes);
           }
         }
-        const int blind = kPeel ? (int)bd.peelDepth : depth;
 #pragma unroll 2
-        for (int d = kMode != kTileRankU8 ? 1 : 0; d < blind; ++d) {
+        for (int d = kMode != kTileRankU8 ? 1 : 0; d < depth; ++d) {
 #pragma unroll
           for (int k = 0; k < K; ++k) {
             const U32x2 node = LdsLoadNode(addr[k]);
@@ -337,31 +393,55 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
             addr[k] = (node.y >> 16) + (left ? 0u : kNodeBytes);
           }
         }
-        if (kPeel) { // the rest only while some lane of the wave still moves (leaves point at themselves)
-          for (int d = blind > 1 || kMode == kTileRankU8 ? blind : 1; d < depth; ++d) {
-            bool moved = false;
+        if (kDefer && bd.hasStubs) {
+          // rows on a stub are queued, the others add their leaf; the queue is walked on as soon as it holds a wave's worth
+          float value[K];
+#pragma unroll
+          for (int k = 0; k < K; ++k) value[k] = LdsLoadFloat(addr[k]);
+#pragma unroll
+          for (int k = 0; k < K; ++k) {
+            const bool stub = __builtin_amdgcn_classf(value[k], 0x3); // a stub's value is a NaN (no leaf's is)
+            acc += (double)(stub ? 0.0f : value[k]);
+            const uint64_t who = __ballot(stub);
+            if (who != 0) {
+              const uint32_t before = __builtin_amdgcn_mbcnt_hi((uint32_t)(who >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)who, 0u));
+              // entry: the NaN's payload (index of the node the stub stands for) below the lane's number
+              if (stub) queue[queued + before] = (__float_as_uint(value[k]) & kStubIndexMask) | laneTag;
+              queued += (uint32_t)__builtin_popcountll(who);
+              if (queued >= 64u) TBAMD_WALK_QUEUE
+            }
+          }
+        } else {
+          if (kDump && s.deferTails && bd.hasStubs) {
+            // the dump walks the rows that stand on a stub on at once, each lane for itself, through the tail array
 #pragma unroll
             for (int k = 0; k < K; ++k) {
-              const U32x2 node = LdsLoadNode(addr[k]);
-              const uint32_t off = kMode == kTileF32Bytes || kMode == kTileRankU16 ? (node.y & 0xFFFFu) : (node.y & 0xFFFFu) << 2;
-              bool left;
-              if (IsRankTile(kMode)) left = RankGoesLeft<kMode>(column + off, node.x);
-              else left = LdsLoadFloat(column + off) < AsFloat(node.x);
-              const uint32_t next = (node.y >> 16) + (left ? 0u : kNodeBytes);
-              moved = moved || next != addr[k];
-              addr[k] = next;
+              const float stop = LdsLoadFloat(addr[k]);
+              if (__builtin_amdgcn_classf(stop, 0x3)) {
+                uint32_t at = __float_as_uint(stop) & kStubIndexMask;
+                U32x2 node = tailNodes[at];
+                for (int d = 0; d < s.tailDepth; ++d) {
+                  const bool left = LdsLoadFloat(column + ((node.y & ((1u << kTailFeatureBits) - 1u)) << tileShift)) < AsFloat(node.x);
+                  at = (node.y >> kTailFeatureBits) + (left ? 0u : 1u);
+                  node = tailNodes[at];
+                }
+                acc += (double)AsFloat(node.x);
+                const int tree = slotTree[bd.firstSlot + k];
+                if (lane < valid && tree >= 0) leafIds[row * s.numTrees + tree] = tailOrigin[at];
+                addr[k] = 0; // (the null leaf: adds 0 below and names no tree's node)
+              }
             }
-            if (!__any(moved)) break;
           }
-        }
 #pragma unroll
-        for (int k = 0; k < K; ++k) acc += (double)LdsLoadFloat(addr[k]);
+          for (int k = 0; k < K; ++k) acc += (double)LdsLoadFloat(addr[k]);
+        }
         if (kDump) {
           if (lane < valid) {
 #pragma unroll
             for (int k = 0; k < K; ++k) {
               const int tree = slotTree[bd.firstSlot + k];
-              if (tree >= 0) leafIds[row * s.numTrees + tree] = nodeOrigin[grp.nodeBegin + addr[k] / kNodeBytes];
+              if (tree >= 0 && !(s.deferTails && addr[k] == 0u))
+                leafIds[row * s.numTrees + tree] = nodeOrigin[grp.nodeBegin + addr[k] / kNodeBytes];
             }
           }
         }
@@ -370,6 +450,8 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
     }
     __builtin_amdgcn_s_setprio(0);
   }
+  if (kDefer) // what is still queued is walked on now
+    while (queued > 0u) TBAMD_WALK_QUEUE
 
   if (C > 0) {
     TBAMD_FLUSH_CLASS(C)
@@ -396,6 +478,7 @@ WalkRowsLdsKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes16
   }
 #undef TBAMD_FLUSH_CLASS
 #undef TBAMD_PREFETCH_GROUP
+#undef TBAMD_WALK_QUEUE
 }
 
 // ---------------------------------------------------------------------------
@@ -1204,19 +1287,23 @@ hipError_t LaunchWalkVariant(const WalkParams &p, dim3 grid, dim3 block, size_t 
   hipError_t e = AllowFullLds<&WalkRowsLdsKernel<K, PF, W, V>>();
   if (e != hipSuccess) return e;
   WalkRowsLdsKernel<K, PF, W, V><<<grid, block, ldsBytes, stream>>>(p.x, p.nodes16, p.bundles, p.bundleRoots, p.groups, p.s, p.out, p.classOut,
-                                                                    p.partial, p.leafIds, p.nodeOrigin, p.slotTree);
+                                                                    p.partial, p.leafIds, p.nodeOrigin, p.slotTree,
+                                                                    reinterpret_cast<const U32x2 *>(p.tailNodes), p.tailOrigin);
   return hipGetLastError();
 }
 
 template <int K, int PF, int W>
 hipError_t LaunchWalkKP(const WalkParams &p, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream) {
   if (p.leafIds) { // (the dump kernel walks every bundle to its full depth and leaves the arg-max to the finalize kernel)
-    if (p.s.fuseArgmax) return hipErrorInvalidValue;
+    if (p.s.fuseArgmax || (p.s.deferTails && W != kTileF32Bytes)) return hipErrorInvalidValue;
     return LaunchWalkVariant<K, PF, W, kWalkDump>(p, grid, block, ldsBytes, stream);
   }
   if (p.s.fuseArgmax) return LaunchWalkVariant<K, PF, W, kWalkFuse>(p, grid, block, ldsBytes, stream);
-  // peeled walks are built for the f32 tile with byte offsets only; elsewhere every bundle walks its full depth
-  if (p.peelWalks && W == kTileF32Bytes) return LaunchWalkVariant<K, PF, kTileF32Bytes, kWalkPeel>(p, grid, block, ldsBytes, stream);
+  // deferred tails are built for the f32 tile with byte offsets only (the packer makes stubs for no other plan)
+  if (p.s.deferTails) {
+    if (W != kTileF32Bytes || p.s.numClasses > 0) return hipErrorInvalidValue;
+    return LaunchWalkVariant<K, PF, kTileF32Bytes, kWalkDefer>(p, grid, block, ldsBytes, stream);
+  }
   return LaunchWalkVariant<K, PF, W, kWalkPlain>(p, grid, block, ldsBytes, stream);
 }
 

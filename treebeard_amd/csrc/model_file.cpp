@@ -21,7 +21,7 @@ namespace tbamd {
 namespace {
 
 constexpr char kMagic[8] = {'T', 'B', 'A', 'M', 'D', 'M', 'D', 'L'};
-constexpr uint32_t kVersion = 4;
+constexpr uint32_t kVersion = 5;
 
 struct Writer {
   std::string bytes;
@@ -80,6 +80,7 @@ void SaveCompiledModel(const std::string &path, const Forest &forest, const Laun
   w.Put<int32_t>(plan.tileSize);
   w.Put<int32_t>(plan.tiling);
   w.Put<int32_t>(plan.peelWalks ? 1 : 0);
+  w.Put<int32_t>(plan.deferTails ? 1 : 0);
   w.Put<uint64_t>(forest.trees.size());
   for (const Tree &t : forest.trees) {
     w.Put<int32_t>(t.classId);
@@ -125,6 +126,7 @@ CompiledModel LoadCompiledModel(const std::string &path) {
   m.plan.tileSize = r.Get<int32_t>();
   m.plan.tiling = r.Get<int32_t>();
   m.plan.peelWalks = r.Get<int32_t>() != 0;
+  m.plan.deferTails = r.Get<int32_t>() != 0;
   const uint64_t trees = r.Get<uint64_t>();
   if (trees > bytes.size()) throw Error("model file is truncated");
   m.forest.trees.resize(trees);

@@ -29,7 +29,7 @@ uint32_t PackedModel::PadFeatureOffset() const { return plan.FeatureOffset((uint
 
 size_t PackedModel::RowTileBytes() const {
   if (plan.rankRows16) return (size_t)((numFeatures + 2) / 2) * plan.rowsPerBlock * 4; // pairs of two-byte ranks, pad feature included
-  return (size_t)(numFeatures + 1) * plan.rowsPerBlock * (plan.quantizedRows ? 1 : 4);
+  return (size_t)(numFeatures + 1) * plan.rowsPerBlock * (plan.quantizedRows ? 1 : 4); // (+ the pad feature's column)
 }
 
 size_t PackedModel::LdsBytes() const {
@@ -43,6 +43,10 @@ size_t PackedModel::LdsBytes() const {
   } else if (plan.treeThreads > 1 && numClasses > 0) {
     bytes = (bytes + 7) & ~(size_t)7;
     bytes += (size_t)plan.ThreadsPerBlock() * 8; // classifiers: cross-wave pass behind the row tile
+  }
+  if (plan.deferTails) {
+    bytes = (bytes + 15) & ~(size_t)15;
+    bytes += (size_t)(plan.ThreadsPerBlock() / 64) * kDeferBytesPerWave; // every wave's queue of deferred walks
   }
   return bytes;
 }
@@ -446,6 +450,9 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCou
   if (T < 1 || T > kMaxTileSize)
     throw Error("tile size " + std::to_string(T) + " is not supported: the device kernels walk tiles of 1 to " +
                 std::to_string(kMaxTileSize) + " nodes");
+  if (plan.deferTails && (plan.kernel != LaunchPlan::Kernel::kRowParallelLds || T != 1 || plan.quantizedRows || plan.rankRows16 ||
+                          plan.featureOffsetInWords || forest.numClasses > 0 || !profile))
+    throw Error("deferred tails need a profile and the scalar row-parallel kernel on float32 rows of a model without classes");
   if (T > 1 && (plan.kernel != LaunchPlan::Kernel::kRowParallelLds || plan.quantizedRows || plan.rankRows16))
     throw Error("tile sizes above 1 need the row-parallel kernel on float32 rows");
   if (T > 1 && (plan.featureOffsetInWords || (int64_t)(forest.numFeatures + 1) * plan.rowsPerBlock * 4 > 0x10000))
@@ -456,6 +463,10 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCou
   pm.numFeatures = forest.numFeatures;
   pm.numClasses = forest.numClasses;
   pm.numTrees = (int32_t)forest.trees.size();
+  if (plan.deferTails) { // tail node 0: a leaf of value 0, what a lane without a queue entry walks
+    pm.tailNodes.push_back(DeviceNode{0.0f, (0u << kTailFeatureBits) | (uint32_t)forest.numFeatures});
+    pm.tailOrigin.push_back(-1);
+  }
   const uint64_t padOffset = pm.PadFeatureOffset();
   if (padOffset > 0xFFFFu)
     throw Error("feature offsets do not fit 16 bits for this rowsPerBlock / feature count");
@@ -539,11 +550,14 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCou
   const size_t numTrees = forest.trees.size();
   std::vector<TiledTree> tiled(T > 1 ? numTrees : 0);
   std::vector<int32_t> depth(numTrees), peel(numTrees);
+  std::vector<int32_t> fullDepth(numTrees, 0); // deferred tails: the tree's own depth (depth[] is then where its walk stops)
+  int64_t tailBudget = plan.deferTails && forest.numFeatures + 1 < (1 << kTailFeatureBits) ? (int64_t)kMaxTailNodes - 1 : 0;
   std::vector<uint32_t> units(numTrees);
   for (size_t t = 0; t < numTrees; ++t) {
     const Tree &tree = forest.trees[t];
     const std::vector<int64_t> *hits = profile ? &profile->hits[t] : nullptr;
     std::vector<int32_t> leafLevel(tree.NumNodes(), -1);
+    std::vector<int32_t> nodeLevel; // scalar nodes: the level of every node
     if (T > 1) {
       tiled[t] = TileTree(tree, T, plan.tiling, hits);
       depth[t] = tiled[t].depth;
@@ -564,10 +578,55 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCou
         stack.push_back(tree.left[n]);
         stack.push_back(tree.right[n]);
       }
+      nodeLevel = leafLevel;
       for (size_t i = 0; i < tree.NumNodes(); ++i)
         if (!tree.IsLeaf((int32_t)i)) leafLevel[i] = -1;
     }
     peel[t] = plan.peelWalks && hits ? PeelDepth(*hits, leafLevel, depth[t]) : depth[t];
+    fullDepth[t] = depth[t];
+    if (plan.deferTails) {
+      // Where the lock-step walk of this tree stops.  Costs in cycles of a compute unit per 64 rows: a lock-step
+      // level is a node read (2.5 cycles while the level has at most 32 nodes, 4.3 for 64, 6.0 beyond) and a
+      // feature read (2.4), as measured on MI355X; a deferred walk costs 20 to queue, fetch and hand back plus 20
+      // per step down to the deepest leaf below the stub (a wave of 64 queue entries runs to the deepest of them),
+      // and the stub test costs every row of the tree 2: the values that, of those tried (6 to 150 per step), gave
+      // the shortest kernel times on two models of 1000 and 800 trees.
+      std::vector<double> alive((size_t)depth[t] + 1, 0.0);
+      {
+        std::vector<std::pair<int32_t, int32_t>> stack{{0, 0}};
+        while (!stack.empty()) {
+          auto [n, level] = stack.back();
+          stack.pop_back();
+          if (tree.IsLeaf(n)) continue;
+          alive[(size_t)level] += (*hits)[0] > 0 ? (double)(*hits)[n] / (double)(*hits)[0] : 1.0;
+          stack.push_back({tree.left[n], level + 1});
+          stack.push_back({tree.right[n], level + 1});
+        }
+      }
+      auto levelCost = [](int32_t d) { return (d <= 5 ? 2.5 : d == 6 ? 4.3 : 6.0) + 2.4; };
+      double whole = 0.0;
+      for (int32_t d = 0; d < depth[t]; ++d) whole += levelCost(d);
+      double best = whole, head = 0.0;
+      int32_t cut = depth[t];
+      for (int32_t d = 1; d < depth[t]; ++d) {
+        head += levelCost(d - 1);
+        const double cost = head + 2.0 + alive[(size_t)d] * ((depth[t] - d) * 20.0 + 20.0);
+        if (cost < best && cost < 0.92 * whole) best = cost, cut = d;
+      }
+      bool nanLeaf = false; // (a NaN is what marks a stub)
+      for (size_t i = 0; i < tree.NumNodes(); ++i) nanLeaf = nanLeaf || (tree.IsLeaf((int32_t)i) && tree.value[i] != tree.value[i]);
+      if (cut < depth[t] && tailBudget > 0 && !nanLeaf) {
+        uint32_t above = 0;
+        for (size_t i = 0; i < tree.NumNodes(); ++i)
+          if (nodeLevel[i] <= cut) ++above; // the top of the tree, the cut level's internal nodes as stubs
+        tailBudget -= (int64_t)(tree.NumNodes() - above) + 64;
+        units[t] = above;
+        depth[t] = cut;
+        peel[t] = cut;
+        pm.treesDeferred += 1;
+        pm.deferredEntriesPerRow += alive[(size_t)cut];
+      }
+    }
     pm.lockStepSteps += depth[t];
     if (hits && (*hits)[0] > 0) {
       double steps = 0.0;
@@ -652,6 +711,70 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCou
       }
       return;
     }
+    if (plan.deferTails && depth[t] < fullDepth[t]) {
+      // The walk of this tree stops at level depth[t]: the internal nodes of that level are represented by stubs
+      // (a NaN whose payload is the index of the node itself in the tail array); their subtrees go to the tail
+      // array in global memory, each in level order with siblings adjacent.
+      const int32_t cut = depth[t];
+      std::vector<int32_t> top, cutNodes, where(tree.NumNodes(), -1);
+      {
+        std::vector<std::pair<int32_t, int32_t>> queue{{0, 0}};
+        for (size_t head = 0; head < queue.size(); ++head) {
+          auto [n, level] = queue[head];
+          where[n] = (int32_t)top.size();
+          top.push_back(n);
+          if (tree.IsLeaf(n)) continue;
+          if (level == cut) { cutNodes.push_back(n); continue; }
+          queue.push_back({tree.left[n], level + 1});
+          queue.push_back({tree.right[n], level + 1});
+        }
+      }
+      if (top.size() != units[t]) throw Error("internal error: deferred tree size out of step");
+      std::vector<uint32_t> tailIndex(tree.NumNodes(), 0);
+      for (int32_t first : cutNodes) {
+        std::vector<int32_t> queue{first};
+        for (size_t head = 0; head < queue.size(); ++head) {
+          const int32_t n = queue[head];
+          if (!tree.IsLeaf(n)) { queue.push_back(tree.left[n]); queue.push_back(tree.right[n]); }
+        }
+        const uint32_t begin = (uint32_t)pm.tailNodes.size();
+        if ((size_t)begin + queue.size() > kMaxTailNodes) throw Error("internal error: tail array overflow");
+        for (size_t i = 0; i < queue.size(); ++i) tailIndex[queue[i]] = begin + (uint32_t)i;
+        for (int32_t n : queue) {
+          DeviceNode dn;
+          dn.value = tree.value[n];
+          if (tree.IsLeaf(n)) {
+            dn.meta = (tailIndex[n] << kTailFeatureBits) | (uint32_t)forest.numFeatures; // stays put: the pad feature holds -inf
+          } else {
+            if (tailIndex[tree.right[n]] != tailIndex[tree.left[n]] + 1) throw Error("internal error: siblings not adjacent");
+            dn.meta = (tailIndex[tree.left[n]] << kTailFeatureBits) | (uint32_t)tree.feature[n];
+          }
+          pm.tailNodes.push_back(dn);
+          pm.tailOrigin.push_back(n);
+        }
+      }
+      for (size_t i = 0; i < top.size(); ++i) {
+        const int32_t n = top[i];
+        const uint32_t self = (base + (uint32_t)i) * kNodeBytes;
+        DeviceNode dn;
+        if (tree.IsLeaf(n)) {
+          dn.value = tree.value[n];
+          dn.meta = (self << 16) | (uint32_t)padOffset;
+        } else if (tailIndex[n] != 0) { // a stub: NaN compares false, so the walk takes the "right" child: the stub itself
+          const uint32_t bits = kStubValueBits | tailIndex[n];
+          std::memcpy(&dn.value, &bits, sizeof(bits));
+          dn.meta = ((self - kNodeBytes) << 16) | (uint32_t)padOffset;
+        } else {
+          dn.value = tree.value[n];
+          if (where[tree.right[n]] != where[tree.left[n]] + 1) throw Error("internal error: siblings not adjacent");
+          dn.meta = (((base + (uint32_t)where[tree.left[n]]) * kNodeBytes) << 16) | plan.FeatureOffset((uint32_t)tree.feature[n]);
+        }
+        pm.nodes.push_back(dn);
+        pm.nodeOrigin.push_back(n);
+      }
+      pm.maxTailDepth = std::max<uint32_t>(pm.maxTailDepth, (uint32_t)(fullDepth[t] - cut));
+      return;
+    }
     const LevelOrder lo = MakeLevelOrder(tree);
     for (size_t i = 0; i < lo.order.size(); ++i) {
       const int32_t n = lo.order[i];
@@ -683,7 +806,7 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCou
     // one spare unit keeps room for the alignment pad
     auto freeNodes = [&]() { return groupCapacity - 1 - ((uint32_t)pm.nodes.size() - g.nodeBegin); };
     bool any = false;
-    struct Mark { size_t nodes, slots, next; };
+    struct Mark { size_t nodes, slots, next, tail; };
     std::vector<Mark> marks; // state before each bundle of this group
     const size_t multiple = plan.kernel == LaunchPlan::Kernel::kRowParallelLds ? (size_t)plan.treeThreads : 1;
     while (next < order.size()) {
@@ -703,8 +826,8 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCou
         ++count;
       }
       if (count == 0) break; // group full
-      marks.push_back(Mark{pm.nodes.size(), pm.slotTree.size(), next});
-      b.classId = (uint32_t)cls;
+      marks.push_back(Mark{pm.nodes.size(), pm.slotTree.size(), next, pm.tailNodes.size()});
+      b.classId = (uint16_t)cls;
       b.firstSlot = (uint32_t)pm.slotTree.size();
       for (int k = 0; k < K; ++k) {
         if (k >= count) {
@@ -717,6 +840,7 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCou
         b.root[k] = (uint16_t)(base * kNodeBytes);
         b.depth = std::max<uint32_t>(b.depth, (uint32_t)depth[t]);
         b.peelDepth = std::max<uint32_t>(b.peelDepth, (uint32_t)peel[t]);
+        if (plan.deferTails && depth[t] < fullDepth[t]) b.hasStubs = 1;
         pm.slotTree.push_back(t);
         emitTree(t, base);
       }
@@ -732,6 +856,8 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCou
       pm.nodes.resize(marks[keep].nodes);
       pm.nodeOrigin.resize(marks[keep].nodes);
       pm.slotTree.resize(marks[keep].slots);
+      pm.tailNodes.resize(marks[keep].tail);
+      pm.tailOrigin.resize(marks[keep].tail);
       pm.bundles.resize(g.bundleBegin + keep);
       pm.bundleRoots.resize((size_t)(g.bundleBegin + keep) * K);
       next = marks[keep].next;
@@ -779,47 +905,75 @@ Tree UnpackTree(const PackedModel &pm, int32_t treeIndex) {
     throw Error("tree not found in packed model");
   }
   const int K = pm.plan.interleave;
-  const uint32_t featureStride = pm.plan.FeatureStride();
   for (const DeviceGroup &g : pm.groups)
     for (uint32_t bi = g.bundleBegin; bi < g.bundleBegin + g.bundleCount; ++bi)
       for (int k = 0; k < K; ++k) {
         if (pm.slotTree[pm.bundles[bi].firstSlot + k] != treeIndex) continue;
-        // walk the packed tree breadth first, restoring original node ids
+        // walk the packed tree breadth first, restoring original node ids (a stub stands for the node its value
+        // field points at)
+        // (units of the group's image; a stub stands for a node of the tail array, noted as kTailBit | index)
+        constexpr uint32_t kTailBit = 0x80000000u;
+        auto resolve = [&](uint32_t unit) {
+          const DeviceNode &dn = pm.nodes[g.nodeBegin + unit];
+          uint32_t bits;
+          std::memcpy(&bits, &dn.value, sizeof(bits));
+          const bool stub = pm.plan.deferTails && (dn.meta >> 16) / kNodeBytes + 1 == unit && (bits & ~kStubIndexMask) == kStubValueBits;
+          if (!stub) return unit;
+          return kTailBit | (bits & kStubIndexMask);
+        };
+        auto nodeAt = [&](uint32_t q) -> const DeviceNode & { return q & kTailBit ? pm.tailNodes[q & ~kTailBit] : pm.nodes[g.nodeBegin + q]; };
+        auto originAt = [&](uint32_t q) { return q & kTailBit ? pm.tailOrigin[q & ~kTailBit] : pm.nodeOrigin[g.nodeBegin + q]; };
+        auto leftOf = [&](uint32_t q) -> uint32_t { // the left child (same notation), or q itself on a leaf
+          const DeviceNode &dn = nodeAt(q);
+          if (q & kTailBit) return kTailBit | (dn.meta >> kTailFeatureBits);
+          return resolve((dn.meta >> 16) / kNodeBytes);
+        };
+        auto rightOf = [&](uint32_t q) -> uint32_t {
+          const DeviceNode &dn = nodeAt(q);
+          if (q & kTailBit) return kTailBit | ((dn.meta >> kTailFeatureBits) + 1);
+          return resolve((dn.meta >> 16) / kNodeBytes + 1);
+        };
+        auto isLeaf = [&](uint32_t q) {
+          const DeviceNode &dn = nodeAt(q);
+          return q & kTailBit ? (dn.meta >> kTailFeatureBits) == (q & ~kTailBit) : (dn.meta >> 16) / kNodeBytes == q;
+        };
+        auto featureOf = [&](uint32_t q) -> int32_t {
+          const DeviceNode &dn = nodeAt(q);
+          return q & kTailBit ? (int32_t)(dn.meta & ((1u << kTailFeatureBits) - 1u)) : (int32_t)pm.plan.FeatureOfOffset(dn.meta & 0xFFFFu);
+        };
         Tree tree;
         tree.classId = pm.bundles[bi].classId;
-        std::vector<uint32_t> queue{pm.bundles[bi].root[k] / kNodeBytes};
+        std::vector<uint32_t> queue{resolve(pm.bundles[bi].root[k] / kNodeBytes)};
         size_t total = 0;
         for (size_t head = 0; head < queue.size(); ++head) {
-          const DeviceNode &dn = pm.nodes[g.nodeBegin + queue[head]];
-          total = std::max<size_t>(total, (size_t)pm.nodeOrigin[g.nodeBegin + queue[head]] + 1);
-          const uint32_t child = (dn.meta >> 16) / kNodeBytes;
-          if (child != queue[head]) { queue.push_back(child); queue.push_back(child + 1); }
+          total = std::max<size_t>(total, (size_t)originAt(queue[head]) + 1);
+          if (!isLeaf(queue[head])) { queue.push_back(leftOf(queue[head])); queue.push_back(rightOf(queue[head])); }
         }
         tree.value.assign(total, 0.f);
         tree.feature.assign(total, 0);
         tree.left.assign(total, -1);
         tree.right.assign(total, -1);
         for (uint32_t q : queue) {
-          const DeviceNode &dn = pm.nodes[g.nodeBegin + q];
-          const int32_t me = pm.nodeOrigin[g.nodeBegin + q];
-          const uint32_t child = (dn.meta >> 16) / kNodeBytes;
+          const DeviceNode &dn = nodeAt(q);
+          const int32_t me = originAt(q);
           tree.value[me] = dn.value;
-          if (child != q && pm.plan.quantizedRows) { // rank -> threshold through the binning table
+          const bool leaf = isLeaf(q);
+          if (!leaf && pm.plan.quantizedRows) { // rank -> threshold through the binning table
             uint32_t j;
             std::memcpy(&j, &dn.value, sizeof(j));
-            const int32_t f = (int32_t)((dn.meta & 0xFFFFu) / featureStride);
+            const int32_t f = featureOf(q);
             const int32_t chunk = pm.binChunkFeatures;
             tree.value[me] = pm.binThresholds[((size_t)(f / chunk) * pm.binTableDepth + j) * chunk + (f % chunk)];
           }
-          if (child != q && pm.plan.rankRows16) {
+          if (!leaf && pm.plan.rankRows16) {
             uint32_t j;
             std::memcpy(&j, &dn.value, sizeof(j));
-            tree.value[me] = pm.rankThresholds.at(pm.plan.FeatureOfOffset(dn.meta & 0xFFFFu)).at(j);
+            tree.value[me] = pm.rankThresholds.at((size_t)featureOf(q)).at(j);
           }
-          if (child != q) {
-            tree.feature[me] = (int32_t)pm.plan.FeatureOfOffset(dn.meta & 0xFFFFu);
-            tree.left[me] = pm.nodeOrigin[g.nodeBegin + child];
-            tree.right[me] = pm.nodeOrigin[g.nodeBegin + child + 1];
+          if (!leaf) {
+            tree.feature[me] = featureOf(q);
+            tree.left[me] = originAt(leftOf(q));
+            tree.right[me] = originAt(rightOf(q));
           }
         }
         return tree;

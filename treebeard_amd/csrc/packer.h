@@ -48,6 +48,11 @@ struct LaunchPlan {
   // steps that bring 90 % of the profiled rows to their leaves without looking, then steps on only while some
   // lane of the wave still moves.
   bool peelWalks = false;
+  // How the scalar row-parallel walk on f32 rows (byte offsets, regressors and binary classifiers) peels: the
+  // walk of a tree stops at the level up to which lock step pays; the internal nodes of that level become
+  // stubs, the rows that reach one are queued per wave as (row, node) and walked on densely, 64 queue entries
+  // at a time, whatever trees they come from.  Needs a profile; set by ChoosePlan where the kernel has the form.
+  bool deferTails = false;
 
   int32_t ThreadsPerBlock() const {
     if (kernel == Kernel::kGlobalWalk) return rowsPerBlock;
@@ -91,6 +96,15 @@ struct PackedModel {
   int32_t treesTiledByProfile = 0;
   int64_t lockStepSteps = 0;
   double profiledSteps = 0.0;
+  // plan.deferTails: trees whose walks stop early, and what the profile says a row's deferred walks cost
+  // The subtrees below the stubs: nodes { value; (left child index << kTailFeatureBits) | feature index } with
+  // indices into this array (right = left + 1; a leaf points at itself and tests the pad feature); entry 0 is a
+  // leaf of value 0.  tailOrigin: original node id of every entry (parity side table).
+  std::vector<DeviceNode> tailNodes;
+  std::vector<int32_t> tailOrigin;
+  uint32_t maxTailDepth = 0; // steps the deepest deferred walk takes below its stub
+  int32_t treesDeferred = 0;
+  double deferredEntriesPerRow = 0.0; // queue entries a profiled row makes over the whole forest
   // kGlobalWalk only:
   std::vector<DeviceGlobalNode> globalNodes;
   std::vector<DeviceGlobalTree> globalTrees; // ordered by (class, depth)

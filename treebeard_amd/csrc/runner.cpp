@@ -159,6 +159,10 @@ void InferenceRunner::FreeModel() {
   (void)hipFree(m_dBinTable);
   (void)hipFree(m_dRankFeatures);
   (void)hipFree(m_dRankChunks);
+  (void)hipFree(m_dTailNodes);
+  (void)hipFree(m_dTailOrigin);
+  m_dTailNodes = nullptr;
+  m_dTailOrigin = nullptr;
   m_dRankFeatures = nullptr;
   m_dRankChunks = nullptr;
   (void)hipFree(m_dGlobalNodes);
@@ -191,6 +195,10 @@ void InferenceRunner::UploadModel() {
   m_dNodeOrigin = Upload(m_model.nodeOrigin, "upload node origins");
   m_dSlotTree = Upload(m_model.slotTree, "upload slot table");
   if (m_model.plan.quantizedRows) m_dBinTable = Upload(m_model.binThresholds, "upload threshold table");
+  if (m_model.plan.deferTails) {
+    m_dTailNodes = Upload(m_model.tailNodes, "upload tail nodes");
+    m_dTailOrigin = Upload(m_model.tailOrigin, "upload tail node origins");
+  }
   if (m_model.plan.rankRows16) {
     m_dBinTable = Upload(m_model.rankTables, "upload threshold tables");
     m_dRankFeatures = Upload(m_model.rankFeatures, "upload rank table index");
@@ -336,6 +344,10 @@ WalkParams InferenceRunner::MakeWalkParams(const float *deviceInputs, int64_t ro
   p.s.treeLanes = m_model.plan.treeLanes;
   p.s.initialValue = m_forest.initialValue;
   p.peelWalks = m_model.plan.peelWalks;
+  p.s.deferTails = m_model.plan.deferTails ? 1 : 0;
+  p.s.tailDepth = (int32_t)m_model.maxTailDepth;
+  p.tailNodes = m_dTailNodes;
+  p.tailOrigin = m_dTailOrigin;
   p.directStaging = DirectStaging();
   p.x = deviceInputs;
   p.globalNodes = m_dGlobalNodes;
@@ -601,6 +613,46 @@ void InferenceRunner::TimeKernels(const float *deviceInputs, void *deviceResults
   }
 }
 
+std::unique_ptr<HitCountProfile> InferenceRunner::CollectProfile(const float *deviceInputs, int64_t rows) {
+  std::unique_ptr<HitCountProfile> profile(new HitCountProfile());
+  const size_t T = m_forest.trees.size();
+  profile->numRows = rows;
+  profile->hits.resize(T);
+  for (size_t t = 0; t < T; ++t) profile->hits[t].assign(m_forest.trees[t].NumNodes(), 0);
+  if (rows <= 0 || T == 0) return profile;
+  int32_t *dIds = nullptr;
+  Check(hipMalloc(reinterpret_cast<void **>(&dIds), (size_t)rows * T * sizeof(int32_t)), "allocate leaf ids");
+  std::vector<int32_t> ids((size_t)rows * T);
+  try {
+    DumpLeafIds(deviceInputs, dIds, rows);
+    Check(hipMemcpy(ids.data(), dIds, ids.size() * sizeof(int32_t), hipMemcpyDeviceToHost), "copy leaf ids");
+  } catch (...) {
+    (void)hipFree(dIds);
+    throw;
+  }
+  (void)hipFree(dIds);
+  for (int64_t r = 0; r < rows; ++r)
+    for (size_t t = 0; t < T; ++t) {
+      const int32_t leaf = ids[(size_t)r * T + t];
+      if (leaf < 0 || (size_t)leaf >= profile->hits[t].size()) throw Error("internal error: leaf id outside its tree");
+      ++profile->hits[t][(size_t)leaf];
+    }
+  // internal nodes: the rows that pass through (children before parents in reverse breadth-first order)
+  for (size_t t = 0; t < T; ++t) {
+    const Tree &tree = m_forest.trees[t];
+    std::vector<int32_t> order{0};
+    for (size_t head = 0; head < order.size(); ++head) {
+      const int32_t n = order[head];
+      if (!tree.IsLeaf(n)) { order.push_back(tree.left[n]); order.push_back(tree.right[n]); }
+    }
+    for (size_t k = order.size(); k-- > 0;) {
+      const int32_t n = order[k];
+      if (!tree.IsLeaf(n)) profile->hits[t][(size_t)n] = profile->hits[t][(size_t)tree.left[n]] + profile->hits[t][(size_t)tree.right[n]];
+    }
+  }
+  return profile;
+}
+
 double InferenceRunner::AutoTune(const float *deviceInputs, int64_t rows) {
   void *out = nullptr;
   Check(hipMalloc(&out, std::max<int64_t>(rows, 1) * sizeof(float)), "allocate tuning output");
@@ -636,6 +688,20 @@ double InferenceRunner::AutoTune(const float *deviceInputs, int64_t rows) {
     std::stable_sort(timed.begin(), timed.end(), [](const Timed &a, const Timed &b) { return a.ms < b.ms; });
     if (timed.size() > 4) timed.resize(4);
     timed.push_back(Timed{original, 0.0});
+    // Peeled walks (deferred tails) of the same shapes: they need a hit-count profile; without one from the caller
+    // the rows of this batch are profiled (leaf ids of up to 4096 rows, counted on the host).
+    if (!original.deferTails && m_forest.numClasses == 0 && original.tileSize == 1) {
+      if (!m_profile) m_profile = CollectProfile(deviceInputs, std::min<int64_t>(rows, 4096));
+      const size_t shapes = timed.size();
+      for (size_t i = 0; i < shapes; ++i) {
+        LaunchPlan p = timed[i].plan;
+        p.peelWalks = true;
+        if (DeferTailsFit(m_forest, &p)) {
+          p.deferTails = true;
+          timed.push_back(Timed{p, 0.0});
+        }
+      }
+    }
     for (const Timed &t : timed) {
       double ms = 0;
       if (timePlan(t.plan, 12, &ms) && ms < bestMs) {
@@ -643,6 +709,7 @@ double InferenceRunner::AutoTune(const float *deviceInputs, int64_t rows) {
         best = m_model.plan;
       }
     }
+    m_walk.peelWalks = best.peelWalks;
     Repack(best);
   } catch (...) {
     (void)hipFree(out);
@@ -661,11 +728,11 @@ std::string InferenceRunner::DescribePlan() const {
   if (p.peelWalks) {
     if (p.kernel == LaunchPlan::Kernel::kTreeParallel) peel = "ignored(tree_parallel)";
     else if (p.kernel == LaunchPlan::Kernel::kGlobalWalk) peel = "ignored(global_walk)";
-    else if (p.tileSize > 1) peel = "1";
-    else if (FusesArgmax()) peel = "ignored(fused)";
+    else if (p.tileSize > 1 || p.deferTails) peel = "1";
+    else if (m_forest.numClasses > 0) peel = "ignored(classes)";
     else if (p.quantizedRows || p.rankRows16) peel = "ignored(ranks)";
     else if (p.featureOffsetInWords) peel = "ignored(words)";
-    else peel = "1";
+    else peel = "ignored(lds)"; // the stub column and the queues do not fit beside this plan's tree groups
   }
   os << "kernel="
      << (p.kernel == LaunchPlan::Kernel::kTreeParallel ? "tree_parallel"
@@ -680,7 +747,8 @@ std::string InferenceRunner::DescribePlan() const {
      << " ldsBytes=" << m_model.LdsBytes() << " tileSize=" << p.tileSize << " tiling=" << p.tiling
      << " staging=" << (DirectStaging() ? "direct" : "registers")
      << " peelWalks=" << peel << " treesTiledByProfile=" << m_model.treesTiledByProfile
-     << " lockStepSteps=" << m_model.lockStepSteps << " profiledSteps=" << m_model.profiledSteps;
+     << " lockStepSteps=" << m_model.lockStepSteps << " profiledSteps=" << m_model.profiledSteps
+     << " treesDeferred=" << m_model.treesDeferred << " deferredEntriesPerRow=" << m_model.deferredEntriesPerRow;
   return os.str();
 }
 

@@ -72,8 +72,11 @@ public:
                    double *finalizeMs, double *binMs);
   // Re-packs the model for another launch plan (used by the timed search).
   void Repack(const LaunchPlan &plan);
-  // Timed search over CandidatePlans(); keeps the fastest.  Returns its time in ms.
+  // Timed search over CandidatePlans(); keeps the fastest.  Returns its time in ms.  A runner without a hit-count
+  // profile profiles up to 4096 of the rows itself, so that peeled walks can be among the candidates.
   double AutoTune(const float *deviceInputs, int64_t rows);
+  // Leaf hit counts of `rows` device-resident rows (the reference's probability profile, src/utils/StatsUtils.cpp:10-52).
+  std::unique_ptr<HitCountProfile> CollectProfile(const float *deviceInputs, int64_t rows);
 
   int32_t BatchSize() const { return m_options.batchSize; }
   int32_t RowSize() const { return m_forest.numFeatures; }
@@ -160,6 +163,8 @@ private:
   double *m_dPartial = nullptr;
   size_t m_partialBytes = 0;
   float *m_dBinTable = nullptr;                 // threshold tables of the rank-quantising kernels (one- or two-byte ranks)
+  DeviceNode *m_dTailNodes = nullptr;           // deferred tails: the subtrees below the stubs
+  int32_t *m_dTailOrigin = nullptr;
   RankFeatureDesc *m_dRankFeatures = nullptr;   // two-byte ranks: per-feature table index
   RankChunkDesc *m_dRankChunks = nullptr;
   uint32_t m_rankChunkEntries = 0, m_rankChunkFeatures = 0; // the largest chunk: the ranking kernel's LDS need

@@ -382,6 +382,10 @@ int32_t tbmi_set_plan(intptr_t h, int32_t rowsPerBlock, int32_t treeThreads, int
         if (treeSlices > 0) plan.treeSlices = treeSlices;
         const int64_t words = (int64_t)(r->RowSize() + 1) * plan.rowsPerBlock;
         plan.featureOffsetInWords = words * 4 > 0xFFFF;
+        // peeled walks keep their form where the new shape has room for it (the caller's group size gives up the
+        // stub column's and the queues' share)
+        plan.deferTails = false;
+        if (plan.peelWalks && r->Profile() && plan.tileSize == 1 && DeferTailsFit(r->GetForest(), &plan)) plan.deferTails = true;
         r->Repack(plan);
         return 0;
       },
@@ -395,6 +399,7 @@ int32_t tbmi_set_tree_parallel_plan(intptr_t h, int32_t rowsPerBlock, int32_t tr
         InferenceRunner *r = Runner(h);
         LaunchPlan plan = r->Model().plan;
         plan.kernel = LaunchPlan::Kernel::kTreeParallel;
+        plan.deferTails = false;
         plan.featureOffsetInWords = false;
         plan.quantizedRows = false;
         plan.rankRows16 = false;
@@ -441,6 +446,7 @@ int32_t tbmi_set_quantized_plan(intptr_t h, int32_t treeThreads, int32_t interle
         plan.kernel = LaunchPlan::Kernel::kRowParallelLds;
         plan.quantizedRows = true;
         plan.rankRows16 = false;
+        plan.deferTails = false;
         plan.featureOffsetInWords = false;
         plan.rowsPerBlock = 64;
         plan.treeLanes = 1;
@@ -464,6 +470,7 @@ int32_t tbmi_set_rank16_plan(intptr_t h, int32_t rowsPerBlock, int32_t treeThrea
         plan.kernel = LaunchPlan::Kernel::kRowParallelLds;
         plan.rankRows16 = true;
         plan.quantizedRows = false;
+        plan.deferTails = false;
         plan.featureOffsetInWords = false;
         plan.treeLanes = 1;
         plan.rowsPerBlock = rowsPerBlock > 0 ? rowsPerBlock : 256;

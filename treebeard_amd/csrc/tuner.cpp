@@ -95,7 +95,22 @@ LaunchPlan ChoosePlan(const Forest &forest, int64_t batchSize, const GPUAutoSche
   plan.tileSize = walk.tileSize;
   plan.tiling = walk.tiling;
   plan.peelWalks = walk.peelWalks;
+  plan.deferTails = false;
+  if (walk.peelWalks && DeferTailsFit(forest, &plan)) plan.deferTails = true;
   return plan;
+}
+
+bool DeferTailsFit(const Forest &forest, LaunchPlan *plan) {
+  if (plan->kernel != LaunchPlan::Kernel::kRowParallelLds || plan->tileSize != 1 || plan->quantizedRows || plan->rankRows16 ||
+      plan->featureOffsetInWords || forest.numClasses > 0)
+    return false;
+  // every wave's queue comes out of the tree group's share of LDS
+  const int64_t extra = (int64_t)(plan->ThreadsPerBlock() / 64) * kDeferBytesPerWave + 32;
+  if (forest.numFeatures + 1 >= (1 << kTailFeatureBits)) return false;
+  const int64_t need = (BiggestTreeNodes(forest) + 2) * kNodeBytes;
+  if (plan->groupBytes - extra < std::max<int64_t>(need, 8192)) return false;
+  plan->groupBytes = (int32_t)((plan->groupBytes - extra) & ~15);
+  return true;
 }
 
 namespace {
@@ -340,6 +355,11 @@ std::vector<LaunchPlan> CandidatePlans(const Forest &forest, int64_t batchSize, 
           if (group < need || group < 8192) continue;
           if (base.treeSlices > 1) group = std::min<int64_t>(group, base.groupBytes);
           p.groupBytes = (int32_t)(group & ~15);
+          if (base.deferTails) {
+            p.deferTails = false;
+            if (!DeferTailsFit(forest, &p)) continue;
+            p.deferTails = true;
+          }
           bool dup = false;
           for (auto &q : out)
             dup = dup || (q.rowsPerBlock == p.rowsPerBlock && q.treeThreads == p.treeThreads &&
@@ -354,6 +374,7 @@ std::vector<LaunchPlan> CandidatePlans(const Forest &forest, int64_t batchSize, 
       if (rowTile > 0xFFFF) continue;
       LaunchPlan p = base;
       p.rankRows16 = true;
+      p.deferTails = false;
       p.featureOffsetInWords = false;
       p.rowsPerBlock = rb;
       p.treeThreads = 1024 / rb;

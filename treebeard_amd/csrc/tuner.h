@@ -30,6 +30,11 @@ struct WalkOptions {
 LaunchPlan ChoosePlan(const Forest &forest, int64_t batchSize, const GPUAutoScheduleOptions *overrides,
                       const DeviceLimits &limits, const WalkOptions &walk = WalkOptions());
 
+// Whether `plan` can defer the tails of its walks (LaunchPlan::deferTails: the scalar row-parallel kernel on an f32
+// tile with byte offsets, a model without classes); when it can, the plan's tree groups give up the LDS the stub
+// feature's column and the waves' queues take.  The caller sets the flag.
+bool DeferTailsFit(const Forest &forest, LaunchPlan *plan);
+
 // Candidate plans for the timed search (the analytic choice comes first).
 std::vector<LaunchPlan> CandidatePlans(const Forest &forest, int64_t batchSize, const DeviceLimits &limits,
                                        const WalkOptions &walk = WalkOptions());
