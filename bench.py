@@ -48,7 +48,7 @@ def print_lds_read_costs():
 def plan_key(plan):
     """The fields of a plan description that decide which kernel runs and how (what a traffic figure is tied to)."""
     keep = ("kernel", "rowsPerBlock", "treeThreads", "treeLanes", "interleave", "groupBytes", "treeSlices", "quantizedRows",
-            "tileSize", "staging")
+            "rankRows16", "tileSize", "staging", "peelWalks")
     fields = dict(item.split("=", 1) for item in plan.split() if "=" in item)
     return " ".join("%s=%s" % (k, fields[k]) for k in keep if k in fields)
 
@@ -64,6 +64,9 @@ def main():
     ap.add_argument("--group-staging", type=int, default=0, choices=[0, 1, 2],
                     help="how tree groups reach LDS: 0 by rule, 1 through prefetch registers, 2 direct global-to-LDS copies")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pin-plan", default="", metavar="ROWS,THREADS,K,GROUPBYTES,SLICES[,peel][,rank16]",
+                    help="skip the search and pin this shape of the row-parallel kernel (what a tuned run printed as its plan): "
+                         "the profiling commands use it, so that every launch of the traced kernel has the measured shape")
     ap.add_argument("--plan", choices=["tuned", "default"], default="tuned",
                     help="tuned: the library's timed launch-plan search (what the reference's findBestGPUScheduleAndCompileModel "
                          "stands for) picks the plan on this batch before anything is measured; default: the analytic plan")
@@ -100,7 +103,16 @@ def main():
     out = torch.zeros(rows, dtype=torch.int8 if multiclass else torch.float32, device="cuda")
     default_plan = runner.describe_plan()
     default_plan_ms = None
-    if args.plan == "tuned":
+    if args.pin_plan:
+        parts = args.pin_plan.split(",")
+        shape = [int(v) for v in parts[:5]]
+        if "rank16" in parts[5:]:
+            runner.set_rank16_plan(*shape)
+        else:
+            runner.set_plan(*shape)
+        if "peel" in parts[5:]:
+            runner.enable_peeled_walks(dx.data_ptr(), rows)
+    elif args.plan == "tuned":
         runner.time_kernels3(dx.data_ptr(), out.data_ptr(), rows, 5)                     # (clocks ramp up)
         default_plan_ms = sum(runner.time_kernels3(dx.data_ptr(), out.data_ptr(), rows, 10))
         runner.autotune(dx.data_ptr(), rows)
@@ -152,7 +164,8 @@ def main():
     lds_time = lds_bytes_row * rows / (LDS_PEAK_GBS * 1e9)
     binding = "lds" if lds_time > hbm_time else "hbm"
     plan = runner.describe_plan()
-    quantized = "quantizedRows=1" in plan
+    quantized = "quantizedRows=1" in plan or "rankRows16=1" in plan       # a ranking kernel runs in front of the walk
+    plan_fields = dict(item.split("=", 1) for item in plan.split() if "=" in item)
     kernel = ("WalkRowsTiledKernel" if " tileSize=1 " not in plan else "WalkRowsLdsKernel") if "rows_lds" in plan else \
         ("WalkGlobalKernel" if "global_walk" in plan else "WalkTreeParallelKernel")
     # the rank-quantised path reads the f32 rows in its binning kernel: both kernels count for the HBM roofline
@@ -186,7 +199,8 @@ def main():
     if lds_measured and binding == "lds":
         per_level = 8.0 / (lds_measured["b64"] * 1e9) + 4.0 / (lds_measured["b32"] * 1e9)
         per_leaf = 4.0 / (lds_measured["b32"] * 1e9)
-        depth_sum = float(sum(forest.depth(t) for t in range(forest.num_trees)))
+        # (peeled walks stop trees early: the plan says how many levels its lock-step walk takes per row)
+        depth_sum = float(plan_fields.get("lockStepSteps") or sum(forest.depth(t) for t in range(forest.num_trees)))
         visited_ms = rows * (steps_per_row * per_level + forest.num_trees * per_leaf) * 1e3
         lockstep_ms = rows * (depth_sum * per_level + forest.num_trees * per_leaf) * 1e3
         lds_floor = {"visited_nodes_ms": visited_ms, "frac_of_visited_floor": visited_ms / walk_ms,
@@ -221,7 +235,7 @@ def main():
     roofline = dict(lds_view if binding == "lds" else hbm_view)
     roofline.update({"traffic": traffic, "traffic_source": "profiles/hbm_traffic.json (rocprofv3 FETCH_SIZE + WRITE_SIZE "
                                                            "of this command, scaled by a plain copy)" if traffic else traffic_note,
-                     "kernel": ("BinRowsKernel+" if quantized else "") + kernel,
+                     "kernel": ("RankRows16Kernel+" if "rankRows16=1" in plan else "BinRowsKernel+" if quantized else "") + kernel,
                      "kernel_ms": hbm_ms if binding == "hbm" else walk_ms,
                      "walk_ms": walk_ms, "finalize_ms": fin_ms, "bin_ms": bin_ms, "path_ms": path_ms})
 
@@ -232,8 +246,8 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": cfg.name, "rows": rows, "trees": forest.num_trees, "features": cfg.num_features,
                    "objective": cfg.objective, "plan": plan,
-                   "plan_source": "timed search over launch plans on this batch (tbmi_autotune)" if args.plan == "tuned"
-                   else "analytic default", "default_plan": default_plan, "default_plan_path_ms": default_plan_ms},
+                   "plan_source": "pinned (--pin-plan %s)" % args.pin_plan if args.pin_plan
+                   else "timed search over launch plans on this batch (tbmi_autotune)" if args.plan == "tuned" else "analytic default", "default_plan": default_plan, "default_plan_path_ms": default_plan_ms},
         "roofline": roofline,
         "roofline_other": hbm_view if binding == "lds" else lds_view,   # the memory roofline that does not bind
     }

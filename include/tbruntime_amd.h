@@ -178,6 +178,11 @@ TBAMD_EXPORT int32_t tbmi_set_global_walk_plan(intptr_t runner, int32_t rowsPerB
 /* Pins the row-parallel kernel on rank-quantised rows (64 rows per block, one byte per feature value). */
 TBAMD_EXPORT int32_t tbmi_set_quantized_plan(intptr_t runner, int32_t treeThreads, int32_t interleave,
                                              int32_t groupBytes, int32_t treeSlices);
+/* Peeled walks (SetPeeledCodeGenForProbabilityBasedTiling, src/runtime/runtime.cpp:309-315) without a profile
+ * file: the library profiles up to 4096 of the given device-resident rows itself (leaf hit counts, as
+ * src/utils/StatsUtils.cpp:10-52 writes them) unless the runner was made with a profile, and re-packs the current
+ * launch plan with peeled walks where the plan has the form (tbmi_describe_plan says `peelWalks=1` or why not). */
+TBAMD_EXPORT int32_t tbmi_enable_peeled_walks(intptr_t runner, const float *deviceInputs, int64_t rows);
 /* Pins the row-parallel kernel on two-byte rank rows: a ranking kernel first replaces every value by the number
  * of its feature's distinct split thresholds that are <= it (exact: every comparison keeps its outcome), laid
  * out so that the walk's row tile takes half the LDS of float32 rows.  For models of up to about 120 features

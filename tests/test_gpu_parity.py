@@ -1130,6 +1130,13 @@ def test_deferred_tails_survive_the_compiled_model_file_and_the_plan_search(synt
     again = treebeard.TreebeardInferenceRunner.FromSOFile(path, "")
     assert again.describe_plan() == runner.describe_plan() and " peelWalks=1 " in again.describe_plan()
     check_against_oracle(again, forest, x[:4096])
+    # peeled walks without a profile file: the library profiles rows on the device itself
+    fresh = make_runner(synth_model(5), rows)
+    dx = torch.from_numpy(x).cuda()
+    torch.cuda.synchronize()
+    fresh.enable_peeled_walks(dx.data_ptr(), rows)
+    assert " peelWalks=1 " in fresh.describe_plan() and int(fresh.describe_plan().split("treesDeferred=")[1].split()[0]) > 100
+    check_against_oracle(fresh, forest, x[:4096])
     # the plan search of a runner without a profile profiles the batch itself and may keep deferred tails; whatever
     # it keeps selects the same leaves
     tuned = make_runner(synth_model(5), rows)

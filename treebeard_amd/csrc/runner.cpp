@@ -653,6 +653,16 @@ std::unique_ptr<HitCountProfile> InferenceRunner::CollectProfile(const float *de
   return profile;
 }
 
+void InferenceRunner::EnablePeeledWalks(const float *deviceInputs, int64_t rows) {
+  if (rows <= 0 || !deviceInputs) throw Error("peeled walks need rows to profile");
+  if (!m_profile) m_profile = CollectProfile(deviceInputs, std::min<int64_t>(rows, 4096));
+  LaunchPlan plan = m_model.plan;
+  plan.peelWalks = true;
+  if (!plan.deferTails && DeferTailsFit(m_forest, &plan)) plan.deferTails = true;
+  Repack(plan);
+  m_walk.peelWalks = true;
+}
+
 double InferenceRunner::AutoTune(const float *deviceInputs, int64_t rows) {
   void *out = nullptr;
   Check(hipMalloc(&out, std::max<int64_t>(rows, 1) * sizeof(float)), "allocate tuning output");

@@ -75,6 +75,9 @@ public:
   // Timed search over CandidatePlans(); keeps the fastest.  Returns its time in ms.  A runner without a hit-count
   // profile profiles up to 4096 of the rows itself, so that peeled walks can be among the candidates.
   double AutoTune(const float *deviceInputs, int64_t rows);
+  // Peeled walks without a profile file: profiles up to 4096 of the given rows on the device (unless the runner
+  // has a profile already) and re-packs the current plan with peeled walks where the plan has the form.
+  void EnablePeeledWalks(const float *deviceInputs, int64_t rows);
   // Leaf hit counts of `rows` device-resident rows (the reference's probability profile, src/utils/StatsUtils.cpp:10-52).
   std::unique_ptr<HitCountProfile> CollectProfile(const float *deviceInputs, int64_t rows);
 

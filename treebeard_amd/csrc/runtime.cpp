@@ -365,6 +365,10 @@ int32_t tbmi_autotune(intptr_t h, const float *in, int64_t rows, double *bestMs)
   return Guard([&] { double ms = Runner(h)->AutoTune(in, rows); if (bestMs) *bestMs = ms; return 0; }, -1);
 }
 
+int32_t tbmi_enable_peeled_walks(intptr_t h, const float *in, int64_t rows) {
+  return Guard([&] { Runner(h)->EnablePeeledWalks(in, rows); return 0; }, -1);
+}
+
 int32_t tbmi_set_plan(intptr_t h, int32_t rowsPerBlock, int32_t treeThreads, int32_t interleave, int32_t groupBytes,
                       int32_t treeSlices) {
   return Guard(

@@ -339,8 +339,8 @@ std::vector<LaunchPlan> CandidatePlans(const Forest &forest, int64_t batchSize, 
   for (int32_t rb : {64, 128, 256, 512})
     for (int32_t tt : {1, 2, 4, 8, 16})
       for (int32_t k : {2, 4, 8})
-        for (int blocksPerCu : {1, 2, 3, 4}) {
-          if (rb * tt > 1024) continue;
+        for (int blocksPerCu : {1, 2, 3, 4, 6, 8}) {
+          if (rb * tt > 1024 || rb * tt * blocksPerCu > 2048) continue; // (a compute unit holds 32 waves)
           bool words = false;
           const int32_t budget = limits.ldsBytesPerBlock / blocksPerCu;
           if (!RowTileFits(forest.numFeatures, rb, budget + 8192, &words)) continue;

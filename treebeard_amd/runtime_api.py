@@ -65,6 +65,7 @@ SIGNATURES = {
     "tbmi_set_global_walk_plan": (c_i32, [c_ip, c_i32, c_i32, c_i32]),
     "tbmi_set_quantized_plan": (c_i32, [c_ip, c_i32, c_i32, c_i32, c_i32]),
     "tbmi_set_rank16_plan": (c_i32, [c_ip, c_i32, c_i32, c_i32, c_i32, c_i32]),
+    "tbmi_enable_peeled_walks": (c_i32, [c_ip, c_vp, c_i64]),
     "tbmi_set_group_staging": (c_i32, [c_ip, c_i32]),
     "tbmi_autotune": (c_i32, [c_ip, c_vp, c_i64, ctypes.POINTER(ctypes.c_double)]),
     "tbmi_set_plan": (c_i32, [c_ip, c_i32, c_i32, c_i32, c_i32, c_i32]),

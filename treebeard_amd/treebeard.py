@@ -352,6 +352,10 @@ class TreebeardInferenceRunner:
         """0 by rule, 1 tree groups through prefetch registers, 2 direct global-to-LDS copies."""
         self._rc(_lib().tbmi_set_group_staging(self.inferenceRunner, mode), "tbmi_set_group_staging")
 
+    def enable_peeled_walks(self, device_inputs_ptr, rows):
+        """Profiles up to 4096 of the device-resident rows and re-packs the current plan with peeled walks."""
+        self._rc(_lib().tbmi_enable_peeled_walks(self.inferenceRunner, device_inputs_ptr, rows), "tbmi_enable_peeled_walks")
+
     def set_rank16_plan(self, rows_per_block=256, tree_threads=0, interleave=4, group_bytes=0, tree_slices=1):
         self._rc(_lib().tbmi_set_rank16_plan(self.inferenceRunner, rows_per_block, tree_threads, interleave, group_bytes,
                                              tree_slices), "tbmi_set_rank16_plan")
