@@ -212,13 +212,14 @@ def main():
     traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(traffic_file):
         with open(traffic_file) as fh:
-            entry = json.load(fh).get("%s@%d" % (cfg.name, rows), {})
-        # the counters were taken on one launch plan: a figure measured on another plan is not this run's traffic
-        if entry.get("plan") == plan_key(plan):
-            traffic = entry.get("bytes_per_launch")
-        elif entry:
-            traffic_note = ("profiles/hbm_traffic.json holds %.4g bytes per launch measured on plan [%s]; this run used [%s]"
-                            % (entry.get("bytes_per_launch", 0), entry.get("plan"), plan_key(plan)))
+            entries = json.load(fh).get("%s@%d" % (cfg.name, rows), [])
+        # the counters were taken on one launch plan each: a figure measured on another plan is not this run's traffic
+        match = [e for e in entries if e.get("plan") == plan_key(plan)]
+        if match:
+            traffic = match[0].get("bytes_per_launch")
+        elif entries:
+            traffic_note = ("profiles/hbm_traffic.json holds figures for the plans %s; this run used [%s]"
+                            % ("; ".join("[%s]" % e.get("plan") for e in entries), plan_key(plan)))
 
     # The roofline that binds this workload (the larger of the two times above): LDS node + feature reads for the
     # narrow models, HBM row streaming for the wide one.  `achieved` = algorithmic bytes per launch / the dominant
