@@ -9,6 +9,7 @@ stand-in for the HIP runtime whose "kernels" interpret the packed model on the C
 hip_host_shim.cpp), driven through host and device entry points of many sizes, plan changes, the plan search
 and the compiled-model file: every buffer the runner sizes and every copy it makes is seen by ASan/UBSan, the
 copier threads by ThreadSanitizer."""
+import concurrent.futures
 import os
 import shutil
 import subprocess
@@ -22,13 +23,26 @@ CSRC = os.path.join(HERE, "..", "treebeard_amd", "csrc")
 HOST_SOURCES = ["forest.cpp", "json_reader.cpp", "xgboost_loader.cpp", "packer.cpp", "tuner.cpp", "model_file.cpp", "host_copy.cpp"]
 
 
+def _compile_and_link(tmp_path, flags, sources, exe):
+    """One g++ per source file, four at a time, then the link: the sanitizer builds are most of these tests' time."""
+    def compile_one(source):
+        obj = str(tmp_path / (os.path.basename(source) + "." + os.path.basename(exe) + ".o"))
+        return obj, subprocess.run(["g++"] + flags + ["-c", source, "-o", obj], capture_output=True, text=True)
+    with concurrent.futures.ThreadPoolExecutor(max_workers=4) as pool:
+        results = list(pool.map(compile_one, sources))
+    for _, built in results:
+        if built.returncode != 0:
+            return built
+    sanitize = [f for f in flags if f.startswith("-fsanitize=")]
+    return subprocess.run(["g++"] + sanitize + [obj for obj, _ in results] + ["-lpthread", "-o", exe], capture_output=True, text=True)
+
+
 @pytest.mark.skipif(shutil.which("g++") is None, reason="needs g++")
 def test_host_code_under_sanitizers(tmp_path, synth_model):
     exe = str(tmp_path / "sanitize_host")
-    cmd = ["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
-           "-fno-omit-frame-pointer", "-I", CSRC, os.path.join(HERE, "native", "sanitize_host.cpp")]
-    cmd += [os.path.join(CSRC, s) for s in HOST_SOURCES] + ["-lpthread", "-o", exe]
-    built = subprocess.run(cmd, capture_output=True, text=True)
+    flags = ["-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
+             "-fno-omit-frame-pointer", "-I", CSRC]
+    built = _compile_and_link(tmp_path, flags, [os.path.join(HERE, "native", "sanitize_host.cpp")] + [os.path.join(CSRC, s) for s in HOST_SOURCES], exe)
     if built.returncode != 0 and "sanitize" in built.stderr:
         pytest.skip("this g++ has no sanitizer runtime")
     assert built.returncode == 0, built.stderr[-2000:]
@@ -44,14 +58,13 @@ RUNNER_SOURCES = HOST_SOURCES + ["onnx_loader.cpp", "runner.cpp", "runtime.cpp"]
 
 def _build_runner_driver(tmp_path, sanitize):
     exe = str(tmp_path / ("sanitize_runner_" + sanitize.split(",")[0]))
-    cmd = ["g++", "-std=c++17", "-O1", "-g", "-fsanitize=" + sanitize, "-fno-omit-frame-pointer",
-           "-D__HIP_PLATFORM_AMD__", "-D__align__(x)=__attribute__((aligned(x)))", "-DHIP_SYMBOL(x)=x",
-           "-I", "/opt/rocm/include", "-I", CSRC,
-           os.path.join(HERE, "native", "sanitize_runner.cpp"), os.path.join(HERE, "native", "hip_host_shim.cpp")]
+    flags = ["-std=c++17", "-O1", "-g", "-fsanitize=" + sanitize, "-fno-omit-frame-pointer",
+             "-D__HIP_PLATFORM_AMD__", "-D__align__(x)=__attribute__((aligned(x)))", "-DHIP_SYMBOL(x)=x",
+             "-I", "/opt/rocm/include", "-I", CSRC]
     if "undefined" in sanitize:
-        cmd.append("-fno-sanitize-recover=undefined")
-    cmd += [os.path.join(CSRC, s) for s in RUNNER_SOURCES] + ["-lpthread", "-o", exe]
-    built = subprocess.run(cmd, capture_output=True, text=True)
+        flags.append("-fno-sanitize-recover=undefined")
+    sources = [os.path.join(HERE, "native", "sanitize_runner.cpp"), os.path.join(HERE, "native", "hip_host_shim.cpp")]
+    built = _compile_and_link(tmp_path, flags, sources + [os.path.join(CSRC, s) for s in RUNNER_SOURCES], exe)
     if built.returncode != 0 and ("sanitize" in built.stderr or "hip/hip_runtime" in built.stderr):
         pytest.skip("this g++ has no sanitizer runtime, or the HIP headers are missing")
     assert built.returncode == 0, built.stderr[-3000:]
@@ -73,7 +86,7 @@ def _wide_model(tmp_path):
 @pytest.mark.skipif(shutil.which("g++") is None, reason="needs g++")
 def test_runner_under_address_sanitizer(tmp_path, synth_model):
     exe = _build_runner_driver(tmp_path, "address,undefined")
-    args = [_wide_model(tmp_path), "8300", synth_model(4), "300", synth_model(3), "1500", synth_model(1), "20000"]
+    args = [_wide_model(tmp_path), "8300", synth_model(4), "300", synth_model(3), "300", synth_model(1), "9000"]
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", TMPDIR=str(tmp_path))
     run = subprocess.run([exe] + args, capture_output=True, text=True, env=env, timeout=900)
     assert run.returncode == 0, (run.stdout + run.stderr)[-4000:]

@@ -1274,12 +1274,19 @@ __global__ void __launch_bounds__(256) FinalizeWideKernel(const FinalizeParams p
   if (lane == 0) p.partial[((int64_t)p.treeSlices * p.rows + row) * Cn + c] = margin - p.initialValue;
 }
 
-// The ceiling on dynamic LDS is an attribute of each kernel: it is raised once per kernel, to the whole
-// 160 KB, instead of on every launch (a runtime call that small batches would pay for each time).
+// The ceiling on dynamic LDS is an attribute of each kernel on each device: it is raised once per kernel and
+// device, to the whole 160 KB, instead of on every launch (a runtime call that small batches would pay for each
+// time).  Two threads that meet here for the first time both make the call, which is harmless.
 template <auto Kernel> hipError_t AllowFullLds() {
-  static const hipError_t status =
-      hipFuncSetAttribute(reinterpret_cast<const void *>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-  return status;
+  constexpr int kMaxDevices = 64;
+  static signed char raised[kMaxDevices] = {};
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return e;
+  if (device >= 0 && device < kMaxDevices && raised[device]) return hipSuccess;
+  e = hipFuncSetAttribute(reinterpret_cast<const void *>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  if (e == hipSuccess && device >= 0 && device < kMaxDevices) raised[device] = 1;
+  return e;
 }
 
 template <int K, int PF, int W, int V>

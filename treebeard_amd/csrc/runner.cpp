@@ -99,8 +99,11 @@ void InferenceRunner::InitDevice() {
   int deviceCount = 0;
   if (hipGetDeviceCount(&deviceCount) != hipSuccess || deviceCount == 0)
     throw Error("no HIP device available: this library has no CPU fallback");
+  // A runner belongs to the device that is current when it is made: its limits, model and workspace are that
+  // device's, and its calls must be made with the same device current.
+  Check(hipGetDevice(&m_device), "hipGetDevice");
   hipDeviceProp_t prop;
-  Check(hipGetDeviceProperties(&prop, 0), "hipGetDeviceProperties");
+  Check(hipGetDeviceProperties(&prop, m_device), "hipGetDeviceProperties");
   m_limits.computeUnits = prop.multiProcessorCount;
   m_limits.ldsBytesPerBlock = (int32_t)std::min<size_t>(prop.sharedMemPerBlock, 160 * 1024);
   // Set-up: the no-allocation entry point finds its array's address ready.  A failure here is that entry
@@ -696,7 +699,7 @@ double InferenceRunner::AutoTune(const float *deviceInputs, int64_t rows) {
       if (timePlan(cand, 3, &ms)) timed.push_back(Timed{m_model.plan, ms});
     }
     std::stable_sort(timed.begin(), timed.end(), [](const Timed &a, const Timed &b) { return a.ms < b.ms; });
-    if (timed.size() > 4) timed.resize(4);
+    if (timed.size() > 6) timed.resize(6);
     timed.push_back(Timed{original, 0.0});
     // Peeled walks (deferred tails) of the same shapes: they need a hit-count profile; without one from the caller
     // the rows of this batch are profiled (leaf ids of up to 4096 rows, counted on the host).
@@ -712,13 +715,24 @@ double InferenceRunner::AutoTune(const float *deviceInputs, int64_t rows) {
         }
       }
     }
-    for (const Timed &t : timed) {
-      double ms = 0;
-      if (timePlan(t.plan, 12, &ms) && ms < bestMs) {
-        bestMs = ms;
-        best = m_model.plan;
+    // The finalists take turns, three passes of eight launches each, and a plan is judged by its best pass: the
+    // clock of the device drifts while it warms up, and a plan timed once, early, would be judged by that.
+    std::vector<double> bestPass(timed.size(), 1e300);
+    for (int pass = 0; pass < 3; ++pass)
+      for (size_t i = 0; i < timed.size(); ++i) {
+        double ms = 0;
+        if (bestPass[i] < 0 || !timePlan(timed[i].plan, 8, &ms)) {
+          bestPass[i] = -1; // a plan that failed once is out
+          continue;
+        }
+        bestPass[i] = std::min(bestPass[i], ms);
+        timed[i].plan = m_model.plan;
       }
-    }
+    for (size_t i = 0; i < timed.size(); ++i)
+      if (bestPass[i] >= 0 && bestPass[i] < bestMs) {
+        bestMs = bestPass[i];
+        best = timed[i].plan;
+      }
     m_walk.peelWalks = best.peelWalks;
     Repack(best);
   } catch (...) {

@@ -142,6 +142,7 @@ private:
   CompilerOptions m_options;
   DeviceLimits m_limits;
   PackedModel m_model;
+  int m_device = 0; // the device that was current at construction
   hipStream_t m_stream = nullptr;
   hipStream_t m_copyStream = nullptr; // host-buffer entry point: copies of the next piece overlap the kernels
   static constexpr int kMaxPieces = 64;
