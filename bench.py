@@ -113,8 +113,10 @@ def main():
         if "peel" in parts[5:]:
             runner.enable_peeled_walks(dx.data_ptr(), rows)
     elif args.plan == "tuned":
-        runner.time_kernels3(dx.data_ptr(), out.data_ptr(), rows, 5)                     # (clocks ramp up)
-        default_plan_ms = sum(runner.time_kernels3(dx.data_ptr(), out.data_ptr(), rows, 10))
+        # the analytic plan's own time, for comparison: after enough launches for the clocks to have ramped up, the
+        # better of two passes (the search judges its finalists the same way)
+        runner.time_kernels3(dx.data_ptr(), out.data_ptr(), rows, 40)
+        default_plan_ms = min(sum(runner.time_kernels3(dx.data_ptr(), out.data_ptr(), rows, 10)) for _ in range(2))
         runner.autotune(dx.data_ptr(), rows)
     if args.copy_calibration:
         # a plain device copy of known size: scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run
