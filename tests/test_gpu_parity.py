@@ -896,6 +896,47 @@ def test_random_forests_and_plans(tmp_path, seed):
     check_against_oracle(runner, forest, x)
 
 
+@pytest.mark.parametrize("seed", range(120))
+def test_random_forests_tiles_and_peeled_walks(tmp_path, seed):
+    """The same differential run over the tiled walk (tile sizes 2 to 8, uniform and profile-driven tiling, peeled or
+    not) and over the scalar walk with deferred tails (profile from a file or taken by the library from device rows)."""
+    rng = np.random.Generator(np.random.PCG64(19000 + seed))
+    path = tmp_path / "m.json"
+    features = _random_forest_file(rng, path)
+    forest = model_io.load_xgboost_json(path)
+    rows = int(rng.choice([1, 33, 64, 129, 500, 2049, 6000]))
+    x = np.round(rng.normal(size=(rows, features)), 1).astype(np.float32)
+    x[rng.random(x.shape) < 0.01] = np.inf
+    x[rng.random(x.shape) < 0.01] = -np.inf
+    shifted = np.round(rng.normal(loc=-0.8, size=(700, features)), 1).astype(np.float32)     # the profiled rows: skewed walks
+    profile = write_profile(tmp_path / "profile.csv", forest, cpu_oracle.leaf_ids(forest, shifted))
+    multiclass = forest.num_classes > 0
+    tile = int(rng.choice([1, 1, 2, 3, 4, 5, 6, 7, 8]))
+    tiling = int(rng.integers(0, 3))
+    peel = bool(rng.random() < 0.6)
+    try:
+        runner = make_tiled_runner(path, rows, tile, tiling, profile if (tiling or peel) else "", peel, multiclass)
+    except RuntimeError as error:        # rows too wide for the tiled walk's row tile
+        assert tile > 1 and "tile" in str(error), str(error)
+        return
+    check_against_oracle(runner, forest, x)
+    if tile == 1 and rng.random() < 0.5:
+        fresh = make_runner(path, rows)
+        dx = torch.from_numpy(shifted).cuda()
+        torch.cuda.synchronize()
+        try:
+            fresh.enable_peeled_walks(dx.data_ptr(), shifted.shape[0])
+        except RuntimeError:
+            pass                         # (a plan without the row-parallel kernel)
+        check_against_oracle(fresh, forest, x)
+    try:
+        rb = int(rng.choice([64, 128, 256]))
+        runner.set_plan(rb, int(rng.choice([1, 2, 4, 8])), int(rng.choice([1, 2, 4])), 0, int(rng.integers(0, 6)))
+    except RuntimeError:
+        pass
+    check_against_oracle(runner, forest, x)
+
+
 def test_lds_micro_benchmark_reports_plausible_rates():
     """The bench-only library (libtbamd_bench.so, not part of the runtime library) that bench.py quotes."""
     from treebeard_amd.runtime_api import lds_read_bandwidth
