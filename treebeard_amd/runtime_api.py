@@ -4,6 +4,13 @@ Counterpart of the reference's `TreebeardAPI` (src/python/treebeard_runtime_api.
 loads the runtime library that sits next to this file and declares argument and
 return types of every entry point.  There is no fallback: a missing library is
 an error.
+
+In a process that also uses PyTorch-ROCm, import torch before the first call that
+loads this library.  The library links against the system's libamdhip64; a torch
+wheel brings a HIP runtime of its own.  With torch loaded first the dynamic linker
+gives this library torch's copy and the process holds one runtime; loaded the other
+way round the process holds two, and torch then reports that no GPU is available
+(measured on MI355X with ROCm 7.2 beside a ROCm 7.0 torch wheel).
 """
 import ctypes
 import os
