@@ -115,8 +115,10 @@ __device__ __forceinline__ void StageRows(const float *__restrict__ src, int val
 // ---------------------------------------------------------------------------
 // Row-parallel walk.  The block owns `rowsPerBlock` rows, kept transposed in
 // LDS (feature-major) so that lane i always reads bank i%64 no matter which
-// feature its node tests.  Trees are streamed through LDS one group at a time;
-// the next group is fetched into registers while the current one is walked.
+// feature its node tests.  Trees are streamed through LDS one group at a time:
+// either the next group is fetched into registers while the current one is walked
+// (PF > 0), or the group is copied by direct global-to-LDS loads between the two
+// barriers of its round while the compute unit's other blocks walk (PF == 0).
 // A lane walks K trees at a time in lock step: all lanes take `depth` steps and
 // leaves hold the walk in place (see device_model.h), so the loop body has no
 // leaf test and no divergence.  `treeThreads` lanes (in different waves) share
