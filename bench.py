@@ -261,14 +261,13 @@ def main():
         # one tree at a time inside a chunk, f32 accumulation.  Timed on a bounded sample of the same batch.
         threads = cpu_oracle.max_threads()
         order = np.argsort([forest.depth(t) for t in range(forest.num_trees)], kind="stable").astype(np.int32)
+        tiled = cpu_oracle.TiledForest(forest, 8)
         if multiclass:
-            run = lambda n: cpu_oracle.predict(forest, x[:n], threads=threads)[0]
-            what = "scalar walk, rows split over %d threads (the tiled schedule has no multiclass form here)" % threads
+            run = lambda n: tiled.predict_tree_outer_multiclass(x[:n], tree_order=order, threads=threads)[0].astype(np.float32)
         else:
-            tiled = cpu_oracle.TiledForest(forest, 8)
             run = lambda n: tiled.predict_tree_outer(x[:n], tree_order=order, threads=threads)
-            what = ("uniform tiling, tile size 8, sparse layout + LUT, depth-ordered trees, one tree at a time, "
-                    "batch split over %d threads" % threads)
+        what = ("uniform tiling, tile size 8, sparse layout + LUT, depth-ordered trees, one tree at a time, "
+                "batch split over %d threads%s" % (threads, ", f32 class sums and the generated code's arg-max" if multiclass else ""))
         probe = min(rows, 4096)
         run(probe)
         t0 = time.perf_counter()

@@ -184,6 +184,22 @@ class TiledForest:
         return out
 
 
+    def predict_tree_outer_multiclass(self, x, tree_order=None, threads=0):
+        """Class ids (int8) and f32 class sums of the multithreaded tree-at-a-time schedule on a multiclass forest."""
+        assert self.forest.num_classes > 0
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        out = np.empty(x.shape[0], dtype=np.int8)
+        sums = np.empty((x.shape[0], self.forest.num_classes), dtype=np.float32)
+        order = None if tree_order is None else np.ascontiguousarray(tree_order, dtype=np.int32)
+        class_id = np.ascontiguousarray(self.forest.class_id, dtype=np.int32)
+        self._L.tiled_predict_tree_outer_multiclass(self.h, _ptr(x), ctypes.c_int64(x.shape[0]),
+                                                    ctypes.c_float(self.forest.initial_value),
+                                                    ctypes.c_int32(self.forest.num_classes), _ptr(class_id), _ptr(out),
+                                                    _ptr(sums), _ptr(order) if order is not None else None,
+                                                    ctypes.c_int32(threads or max_threads()))
+        return out, sums
+
+
 def lut_for_shape(left_slot, right_slot, tile_size):
     """LUT row (2^tile_size entries) of a tile whose nodes (level order) have the given children slots (-1: exit)."""
     l = np.ascontiguousarray(left_slot, dtype=np.int32)

@@ -339,6 +339,44 @@ void tiled_predict_tree_outer(const tiled_forest_t *f, const float *x, int64_t r
   }
 }
 
+/*
+ * The same schedule for a multiclass forest: every chunk keeps f32 class sums [rows][C], each filled with the
+ * initial value before the trees are added (src/reduction/LowerReduceOps.cpp:1459-1470), tree t adds its leaf to
+ * class class_id[t] (GenerateMultiClassAccumulate, src/mlir/LowerToMidLevelIR.cpp:405-429), and the class id is
+ * the generated code's arg-max: running maximum from -inf / class 0, replaced unless `max > cur`, so exact ties go
+ * to the larger class id (LowerReduceOps.cpp:148-187).  `sums` may be NULL; `out_class` takes the ids as int8.
+ */
+void tiled_predict_tree_outer_multiclass(const tiled_forest_t *f, const float *x, int64_t rows, float initial_value,
+                                         int32_t num_classes, const int32_t *class_id, int8_t *out_class, float *sums,
+                                         const int32_t *tree_order, int32_t threads) {
+  const int32_t NT = f->num_trees, F = f->num_features, C = num_classes;
+  const int avx = have_avx2(f);
+  if (threads < 1) threads = 1;
+#pragma omp parallel for num_threads(threads) schedule(static)
+  for (int32_t k = 0; k < threads; ++k) {
+    const int64_t lo = rows * k / threads, hi = rows * (k + 1) / threads;
+    if (hi <= lo) continue;
+    float *acc = sums ? sums + lo * C : (float *)malloc((size_t)(hi - lo) * (size_t)C * sizeof(float));
+    for (int64_t i = 0; i < (hi - lo) * C; ++i) acc[i] = initial_value;
+    for (int32_t i = 0; i < NT; ++i) {
+      const int32_t t = tree_order ? tree_order[i] : i;
+      const float *leaves = f->leaf_value + f->leaf_begin[t];
+      const int32_t c = class_id[t];
+      for (int64_t r = lo; r < hi; ++r) acc[(r - lo) * C + c] += leaves[walk_tiled(f, t, x + r * F, avx)];
+    }
+    for (int64_t r = lo; r < hi; ++r) {
+      float mx = -INFINITY;
+      int32_t idx = 0;
+      for (int32_t c = 0; c < C; ++c) {
+        const float cur = acc[(r - lo) * C + c];
+        if (!(mx > cur)) { mx = cur; idx = c; }
+      }
+      out_class[r] = (int8_t)idx;
+    }
+    if (!sums) free(acc);
+  }
+}
+
 /* LUT row of an explicitly given shape (for the documented known-answer checks). */
 void tiled_lut_for_shape(int32_t n, const int32_t *left_slot, const int32_t *right_slot, int32_t tile_size,
                          int8_t *lut_row) {

@@ -14,6 +14,7 @@ import pytest
 import scipy.special
 
 from oracle import cpu_oracle, model_io
+from treebeard_amd import synth
 
 from conftest import BENCHMARK_XGB, GOLDEN, benchmark_csv, benchmark_model, random_models
 
@@ -248,6 +249,31 @@ def test_tile_shapes_and_lut_known_answers():
         assert found <= catalan
         if tile_size <= 4:
             assert found == catalan
+
+
+def test_tiled_multithreaded_schedule_on_a_multiclass_forest(tmp_path, synth_model):
+    """Class sums = the scalar walker's per-class sums (f32 order tolerance), class ids = the generated code's arg-max of
+    them, exact ties included (two identical trees voting for classes 1 and 3: the larger id wins)."""
+    forest = model_io.load_xgboost_json(synth_model(3))
+    x = synth.CONFIGS[3].batch_rows(700, seed_offset=4)
+    order = np.argsort([forest.depth(t) for t in range(forest.num_trees)], kind="stable").astype(np.int32)
+    ids, sums = cpu_oracle.TiledForest(forest, 8).predict_tree_outer_multiclass(x, tree_order=order, threads=3)
+    pred, margins = cpu_oracle.predict(forest, x)
+    np.testing.assert_allclose(sums, margins, rtol=1e-5, atol=1e-6)
+    np.testing.assert_array_equal(ids, cpu_oracle.argmax_generated(sums))
+    assert (ids == pred.astype(np.int8)).mean() > 0.999           # (f32 against f64 sums: only near-ties may differ)
+    rng = np.random.Generator(np.random.PCG64(3))
+    tree = synth._grow_tree(rng, 3, lambda d, s: 1.0, lambda: (int(rng.integers(0, 4)), float(np.round(rng.normal(), 1))),
+                            lambda: float(rng.normal()))
+    path = tmp_path / "ties.json"
+    synth.write_xgboost_json(path, [tree, tree], 4, objective="multi:softmax", num_class=4, tree_info=[1, 3])
+    tied = model_io.load_xgboost_json(path)
+    rows = rng.normal(size=(64, 4)).astype(np.float32)
+    ids, sums = cpu_oracle.TiledForest(tied, 8).predict_tree_outer_multiclass(rows, threads=2)
+    np.testing.assert_array_equal(sums[:, 1], sums[:, 3])
+    positive = sums[:, 1] > tied.initial_value
+    np.testing.assert_array_equal(ids[positive], 3)                # classes 1 and 3 tie above the others: 3
+    np.testing.assert_array_equal(ids[~positive & (sums[:, 1] < tied.initial_value)], 2)   # classes 0 and 2 tie at the initial value: 2
 
 
 def test_tiled_multithreaded_schedule_matches_scalar_schedule():
