@@ -937,6 +937,34 @@ def test_random_forests_tiles_and_peeled_walks(tmp_path, seed):
     check_against_oracle(runner, forest, x)
 
 
+@pytest.mark.parametrize("k,rows", [(1, (1 << 29) + 3), (4, (1 << 20) + (1 << 18) + 5)])
+def test_batches_past_32_bit_offsets(synth_model, k, rows):
+    """Maximum sizes: batches of more than 2^31 elements (17 GB and 10 GB of rows, generated on the device), checked
+    against the oracle on slices at both ends, in the middle and on either side of the rows where the element index
+    passes 2^31 and the byte offset 2^32."""
+    forest = model_io.load_xgboost_json(synth_model(k))
+    features = forest.num_features
+    generator = torch.Generator(device="cuda")
+    generator.manual_seed(40 + k)
+    x = torch.empty((rows, features), dtype=torch.float32, device="cuda")
+    for lo in range(0, rows, 1 << 22):
+        x[lo:lo + (1 << 22)].normal_(generator=generator)
+    runner = make_runner(synth_model(k), rows)
+    out = torch.zeros(rows, dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    runner.run_device(x.data_ptr(), out.data_ptr(), rows)
+    torch.cuda.synchronize()
+    marks = [150, rows // 2, rows - 150, (1 << 31) // features, (1 << 30) // features]
+    for mark in marks:
+        if mark + 150 > rows:
+            continue
+        rows_here = x[mark - 150:mark + 150].cpu().numpy()
+        pred, _ = cpu_oracle.predict(forest, rows_here)
+        np.testing.assert_allclose(out[mark - 150:mark + 150].cpu().numpy(), pred, rtol=RTOL_SUM, atol=0)
+    del x, out
+    torch.cuda.empty_cache()
+
+
 def test_lds_micro_benchmark_reports_plausible_rates():
     """The bench-only library (libtbamd_bench.so, not part of the runtime library) that bench.py quotes."""
     from treebeard_amd.runtime_api import lds_read_bandwidth
