@@ -290,7 +290,7 @@ namespace {
 
 // One tile step of the tiled layout (device_model.h): returns the byte address of the child tile.
 uint32_t TileStepHost(const unsigned char *group, uint32_t groupBytes, uint32_t addr, int T, const float *row, int F,
-                      uint32_t stride) {
+                      uint32_t stride, int hops) {
   const uint32_t bytes = TileBytes(T);
   if (addr % 8 != 0 || addr + bytes > groupBytes) std::abort(); // tile outside the group
   const unsigned char *tile = group + addr;
@@ -303,11 +303,11 @@ uint32_t TileStepHost(const unsigned char *group, uint32_t groupBytes, uint32_t 
     std::memcpy(&links, tile + 48, 8);
     std::memcpy(&base, tile + 56, 2);
     uint32_t slot = 0;
-    for (int hop = 0; hop < 8; ++hop) {
+    for (int hop = 0; hop < hops; ++hop) { // (the kernel follows `hops` links: they must reach a child)
       if (off8[slot] % stride != 0 || (int)(off8[slot] / stride) > F) std::abort();
       const int f = (int)(off8[slot] / stride);
       const float x = f == F ? -INFINITY : row[f];
-      const uint32_t link = (uint32_t)(links >> (8 * slot + (x < thr8[slot] ? 4 : 0))) & 15u;
+      const uint32_t link = (uint32_t)(links >> (4 * slot + (x < thr8[slot] ? 32 : 0))) & 15u;
       if (link >= kTileLinkExit) return base + (link - kTileLinkExit) * bytes;
       slot = link + 1;
     }
@@ -372,8 +372,8 @@ hipError_t LaunchWalkRowsTiled(const WalkParams &p, int tileSize, int interleave
             // the kernel stops early only when no lane moves any more, which leaves every lane where `depth`
             // steps would: the full walk is the specification
             for (uint32_t d = 0; d < bd.depth; ++d)
-              addr = TileStepHost(group, grp.nodeCount * kNodeBytes, addr, T, p.x + row * F, F, (uint32_t)RB * 4u);
-            const uint32_t settled = TileStepHost(group, grp.nodeCount * kNodeBytes, addr, T, p.x + row * F, F, (uint32_t)RB * 4u);
+              addr = TileStepHost(group, grp.nodeCount * kNodeBytes, addr, T, p.x + row * F, F, (uint32_t)RB * 4u, p.s.tileHops);
+            const uint32_t settled = TileStepHost(group, grp.nodeCount * kNodeBytes, addr, T, p.x + row * F, F, (uint32_t)RB * 4u, p.s.tileHops);
             if (settled != addr) std::abort(); // `depth` steps must end on a leaf tile
             float value;
             std::memcpy(&value, group + addr, 4);

@@ -54,11 +54,13 @@
 //      { f32 thr[8]; u16 off[8]; u64 links; u16 childBase; u16 pad[3] }
 //    A table of 256 outcomes does not fit a tile, and one row of the reference's LUT per shape present in a
 //    model (1430 shapes of 256 entries) fits no LDS, so the tile carries its own shape instead: `links` holds
-//    two 4-bit links per slot, nibble 2 s + 1 taken when slot s sends the row left (its outcome bit is set) and
-//    nibble 2 s when it sends it right.  A link below 7 names the next slot (link + 1: slot 0 is nobody's
-//    child), a link of 7 or more the child reached (link - 7, children numbered left to right, 0..8).  The
-//    walk follows at most eight links from slot 0; this is the reference's LUT[shape][outcome] evaluated
-//    instead of stored, so the outcome bit order and the child numbering are the same.  A leaf tile's links
+//    a 4-bit link per slot and outcome, nibble s of the high word taken when slot s sends the row left (its
+//    predicate holds) and nibble s of the low word when it sends it right.  A link below 7 names the next slot
+//    (link + 1: slot 0 is nobody's child), a link of 7 or more the child reached (link - 7, children numbered
+//    left to right, 0..8).  A tile step picks the eight links its comparisons select with one masked insert of
+//    the high word into the low one and follows them from slot 0, as many as the tiles of the model have
+//    levels of nodes; this is the reference's LUT[shape][outcome] evaluated instead of stored, so the outcome
+//    bit order and the child numbering are the same.  A leaf tile's links
 //    all say "child 0" and its childBase is its own address.
 #pragma once
 

@@ -27,6 +27,7 @@ struct WalkScalars {
   // tile then has a column for the stub feature and every wave a queue of deferred walks behind it.
   int32_t deferTails = 0;
   int32_t tailDepth = 0;         // steps the deepest deferred walk takes below its stub
+  int32_t tileHops = 1;          // eight-slot tiles: links a tile step follows at most (levels of nodes inside a tile)
   double initialValue = 0.0;
 };
 

@@ -503,7 +503,7 @@ typedef const __attribute__((address_space(3))) U32x4 *LdsQuadPtr;
 __device__ __forceinline__ U32x4 LdsLoadQuad(uint32_t address) { return *(LdsQuadPtr)(uintptr_t)address; }
 
 template <int T> // 2, 3, 4, or kMaxTileSize for the eight-slot tile of tile sizes 5 to 8
-__device__ __forceinline__ uint32_t TileStep(uint32_t addr, uint32_t column) {
+__device__ __forceinline__ uint32_t TileStep(uint32_t addr, uint32_t column, int hops) {
   static_assert(T >= 2 && (T <= kMaxSelectTile || T == kMaxTileSize), "tile sizes 5 to 8 share the eight-slot tile");
   float thr[T];
   uint32_t off[T];
@@ -536,24 +536,31 @@ __device__ __forceinline__ uint32_t TileStep(uint32_t addr, uint32_t column) {
     select = (uint64_t)q3.x | ((uint64_t)q3.y << 32);
     childBase = q3.z & 0xFFFFu;
   }
-  uint32_t outcome = 0;
-#pragma unroll
-  for (int i = 0; i < T; ++i) {
-    const float x = LdsLoadFloat(column + off[i]);
-    outcome |= (x < thr[i] ? 1u : 0u) << i;
-  }
   if constexpr (T > kMaxSelectTile) {
-    // Follow the tile's links from slot 0: nibble 2 s + 1 when slot s sends the row left, nibble 2 s otherwise; a
-    // link below kTileLinkExit names the next slot, the others the child.  Eight slots: at most eight links.
-    uint32_t link = (uint32_t)(select >> ((outcome & 1u) << 2)) & 15u;
+    // The eight comparisons pick, slot by slot, the link the slot sends its row along: nibble s of the high word
+    // of `select` when slot s sends the row left, nibble s of the low word otherwise (one bit-field insert under a
+    // mask of eight nibbles).  Then the links are followed from slot 0: a link below kTileLinkExit names the next
+    // slot (link + 1), the others the child; a tile holds `hops` levels of nodes, so `hops` links reach a child.
+    uint32_t wentLeft = 0;
 #pragma unroll
-    for (int hop = 1; hop < T; ++hop) {
-      const uint32_t slot = (link + 1u) & 7u;
-      const uint32_t next = (uint32_t)(select >> (slot * 8u + (((outcome >> slot) & 1u) << 2))) & 15u;
+    for (int i = 0; i < T; ++i) {
+      const float x = LdsLoadFloat(column + off[i]);
+      wentLeft |= x < thr[i] ? 0xFu << (4 * i) : 0u;
+    }
+    const uint32_t taken = ((uint32_t)(select >> 32) & wentLeft) | ((uint32_t)select & ~wentLeft);
+    uint32_t link = taken & 15u;
+    for (int hop = 1; hop < hops; ++hop) {
+      const uint32_t next = __builtin_amdgcn_ubfe(taken, (link + 1u) << 2, 4u); // (the field offset wraps at 32 for a link that names a child: ignored below)
       link = link < kTileLinkExit ? next : link;
     }
     return childBase + (link - kTileLinkExit) * TileBytes(T);
   } else {
+    uint32_t outcome = 0;
+#pragma unroll
+    for (int i = 0; i < T; ++i) {
+      const float x = LdsLoadFloat(column + off[i]);
+      outcome |= (x < thr[i] ? 1u : 0u) << i;
+    }
     const uint32_t child = (uint32_t)(select >> (outcome * TileSelectBits(T))) & ((1u << TileSelectBits(T)) - 1u);
     return childBase + child * TileBytes(T);
   }
@@ -661,13 +668,13 @@ WalkRowsTiledKernel(const float *__restrict__ x, const uint4 *__restrict__ nodes
         const int blind = (int)bd.peelDepth;
         for (int d = 0; d < blind; ++d) {
 #pragma unroll
-          for (int k = 0; k < K; ++k) addr[k] = TileStep<T>(addr[k], column);
+          for (int k = 0; k < K; ++k) addr[k] = TileStep<T>(addr[k], column, s.tileHops);
         }
         for (int d = blind; d < depth; ++d) {
           bool moved = false;
 #pragma unroll
           for (int k = 0; k < K; ++k) {
-            const uint32_t next = TileStep<T>(addr[k], column);
+            const uint32_t next = TileStep<T>(addr[k], column, s.tileHops);
             moved = moved || next != addr[k];
             addr[k] = next;
           }

@@ -112,7 +112,8 @@ struct TileInfo {
   int32_t leafNode = -1;                   // leaf tiles: the original leaf
   uint32_t firstChild = 0;                 // tile index (inside the tree) of child 0; own index on a leaf tile
   uint64_t select = 0;                     // child number per outcome word, TileSelectBits() each (tiles of up to 4 nodes)
-  uint64_t links = kLeafTileLinks;         // two 4-bit links per slot (tiles of 5 to 8 nodes, device_model.h)
+  uint64_t links = kLeafTileLinks;         // a 4-bit link per slot and outcome (tiles of 5 to 8 nodes, device_model.h)
+  int32_t hops = 1;                        // links a walk follows inside the tile at most (its levels of nodes)
   int32_t depth = 0;                       // tile steps from this tile down to its deepest leaf
   int32_t level = 0;                       // tile steps from the root tile
 };
@@ -120,6 +121,7 @@ struct TileInfo {
 struct TiledTree {
   std::vector<TileInfo> tiles; // children of a tile are consecutive
   int32_t depth = 0;           // tile steps that bring every row to a leaf tile
+  int32_t hops = 1;            // the most levels of nodes any tile holds
   bool byProfile = false;
 };
 
@@ -288,8 +290,10 @@ TiledTree TileTree(const Tree &tree, int T, int tiling, const std::vector<int64_
       tile.links = 0;
       for (int slot = 0; slot < kMaxTileSize; ++slot) {
         const uint64_t left = slot < n ? link(leftSlot[slot]) : kTileLinkExit, right = slot < n ? link(rightSlot[slot]) : kTileLinkExit;
-        tile.links |= (right << (8 * slot)) | (left << (8 * slot + 4));
+        tile.links |= (right << (4 * slot)) | (left << (32 + 4 * slot));
       }
+      for (int i = 0; i < n; ++i) tile.hops = std::max(tile.hops, nodeDepth[tile.members[i]] - nodeDepth[tile.members[0]] + 1);
+      out.hops = std::max(out.hops, tile.hops);
     }
     tile.firstChild = (uint32_t)roots.size();
     for (int e = 0; e < tile.numExits; ++e) roots.push_back(tile.exits[e]);
@@ -563,6 +567,7 @@ PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCou
       depth[t] = tiled[t].depth;
       units[t] = (uint32_t)tiled[t].tiles.size() * tileUnits;
       pm.treesTiledByProfile += tiled[t].byProfile ? 1 : 0;
+      pm.maxTileHops = std::max(pm.maxTileHops, tiled[t].hops);
       for (const TileInfo &tile : tiled[t].tiles)
         if (tile.count == 0) leafLevel[tile.leafNode] = tile.level;
     } else {

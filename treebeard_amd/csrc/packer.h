@@ -94,6 +94,7 @@ struct PackedModel {
   // one row takes over the whole forest: lock-step (deepest leaf of every tree) and, when a profile was
   // given, what the profiled rows need on average.
   int32_t treesTiledByProfile = 0;
+  int32_t maxTileHops = 1;   // eight-slot tiles: the most levels of nodes any tile holds (links a tile step follows)
   int64_t lockStepSteps = 0;
   double profiledSteps = 0.0;
   // plan.deferTails: trees whose walks stop early, and what the profile says a row's deferred walks cost

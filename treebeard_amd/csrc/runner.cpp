@@ -349,6 +349,7 @@ WalkParams InferenceRunner::MakeWalkParams(const float *deviceInputs, int64_t ro
   p.peelWalks = m_model.plan.peelWalks;
   p.s.deferTails = m_model.plan.deferTails ? 1 : 0;
   p.s.tailDepth = (int32_t)m_model.maxTailDepth;
+  p.s.tileHops = m_model.maxTileHops;
   p.tailNodes = m_dTailNodes;
   p.tailOrigin = m_dTailOrigin;
   p.directStaging = DirectStaging();
