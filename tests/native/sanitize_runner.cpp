@@ -10,7 +10,10 @@
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
+#include <cstdint>
 #include <cstring>
+#include <fstream>
+#include <iterator>
 #include <random>
 #include <string>
 #include <vector>
@@ -332,8 +335,56 @@ void DeviceEntryPoints(const Case &c, int64_t rows, int32_t tileSize = 1, int32_
 
 } // namespace
 
+// Compiled-model files with mutated bytes through tbmi_load_compiled_model and, where one loads, through a host call
+// of a few rows: the header's plan, batch size and return type are what a runner is built from.
+static int MutatedCompiledModels(const char *path, int iterations) {
+  std::ifstream in(path, std::ios::binary);
+  const std::vector<char> good((std::istreambuf_iterator<char>(in)), std::istreambuf_iterator<char>());
+  EXPECT(!good.empty(), "cannot read %s", path);
+  const std::string scratch = std::string(std::getenv("TMPDIR") ? std::getenv("TMPDIR") : "/tmp") + "/mutated.tbamd";
+  std::mt19937 rng(13);
+  long loaded = 0;
+  for (int i = 0; i < iterations; ++i) {
+    std::vector<char> bytes = good;
+    if (i > 0) {
+      const int edits = 1 + (int)(rng() % 3);
+      for (int e = 0; e < edits; ++e) {
+        const int32_t words[] = {0, 1, -1, 2, 3, 7, 8, 9, 63, 64, 65, 255, 1000, 1024, 65536, 1 << 20, 1 << 30, INT32_MIN};
+        const int32_t w = words[rng() % 18];
+        const size_t limit = rng() % 4 ? std::min<size_t>(bytes.size(), 140) : bytes.size(); // mostly the header
+        const size_t p = (rng() % limit) & ~(size_t)3;
+        std::memcpy(bytes.data() + p, &w, std::min<size_t>(4, bytes.size() - p));
+      }
+    }
+    {
+      std::ofstream out(scratch, std::ios::binary | std::ios::trunc);
+      out.write(bytes.data(), (std::streamsize)bytes.size());
+    }
+    const intptr_t runner = tbmi_load_compiled_model(scratch.c_str(), 0);
+    if (!runner) {
+      EXPECT(i > 0, "the intact compiled model was refused: %s", tbmi_last_error());
+      continue;
+    }
+    ++loaded;
+    const int32_t F = GetRowSize(runner);
+    EXPECT(F > 0 && F < (1 << 20), "row size %d of a loaded model", F);
+    const int64_t rows = 70;
+    std::vector<float> x((size_t)rows * F, 0.25f);
+    std::vector<unsigned char> out((size_t)rows * (size_t)tbmi_result_bytes(runner), 0xEE); // exactly what the call may write
+    (void)tbmi_run_host(runner, x.data(), out.data(), rows); // may be refused; must not overrun
+    DeleteInferenceRunner(runner);
+  }
+  std::printf("mutated compiled models: %ld of %d loaded\n", loaded, iterations);
+  return gFailures;
+}
+
 int main(int argc, char **argv) {
-  // argv: pairs of <model.json> <rows>
+  // argv: pairs of <model.json> <rows>, or --mutate <compiled model> <iterations>
+  if (argc == 4 && std::strcmp(argv[1], "--mutate") == 0) {
+    if (int rc = MutatedCompiledModels(argv[2], std::atoi(argv[3]))) return rc;
+    std::printf("ok\n");
+    return 0;
+  }
   std::mt19937 rng(7);
   std::normal_distribution<float> normal(0.f, 1.f);
   for (int a = 1; a + 1 < argc; a += 2) {

@@ -38,14 +38,8 @@ def _compile_and_link(tmp_path, flags, sources, exe):
 
 
 @pytest.mark.skipif(shutil.which("g++") is None, reason="needs g++")
-def test_host_code_under_sanitizers(tmp_path, synth_model):
-    exe = str(tmp_path / "sanitize_host")
-    flags = ["-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
-             "-fno-omit-frame-pointer", "-I", CSRC]
-    built = _compile_and_link(tmp_path, flags, [os.path.join(HERE, "native", "sanitize_host.cpp")] + [os.path.join(CSRC, s) for s in HOST_SOURCES], exe)
-    if built.returncode != 0 and "sanitize" in built.stderr:
-        pytest.skip("this g++ has no sanitizer runtime")
-    assert built.returncode == 0, built.stderr[-2000:]
+def test_host_code_under_sanitizers(tmp_path, synth_model, host_driver):
+    exe = host_driver
     models = [synth_model(k) for k in (1, 2, 3, 4, 5)]
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", TMPDIR=str(tmp_path))
     run = subprocess.run([exe] + models, capture_output=True, text=True, env=env, timeout=900)
@@ -71,6 +65,62 @@ def _build_runner_driver(tmp_path, sanitize):
     return exe
 
 
+@pytest.mark.skipif(shutil.which("g++") is None, reason="needs g++")
+def test_loaders_survive_mutated_files(tmp_path, host_driver):
+    """Flipped bytes, overwritten words, cut and doubled pieces in an XGBoost JSON file, an ONNX file and a compiled-model
+    file: every mutant is refused with an error or loads into a forest that validates and packs, under ASan + UBSan."""
+    import sys
+    import numpy as np
+    sys.path.insert(0, HERE)
+    from onnx_writer import write_onnx
+    rng = np.random.Generator(np.random.PCG64(11))
+    trees = [synth._grow_tree(rng, 4, lambda d, s: 0.8, lambda: (rng.integers(0, 6), np.round(rng.normal(), 2)),
+                              lambda: rng.normal(0.0, 0.1)) for _ in range(6)]
+    json_path = str(tmp_path / "small.json")
+    synth.write_xgboost_json(json_path, trees, 6, objective="binary:logistic")
+    onnx_path = str(tmp_path / "small.onnx")
+    write_onnx(onnx_path, [(t.value, t.feature, t.left, t.right) for t in trees], post_transform="LOGISTIC")
+    exe = str(tmp_path / "mutate_loaders")
+    flags = ["-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
+             "-fno-omit-frame-pointer", "-I", CSRC]
+    sources = [os.path.join(HERE, "native", "mutate_loaders.cpp")] + [os.path.join(CSRC, s) for s in HOST_SOURCES + ["onnx_loader.cpp"]]
+    built = _compile_and_link(tmp_path, flags, sources, exe)
+    if built.returncode != 0 and "sanitize" in built.stderr:
+        pytest.skip("this g++ has no sanitizer runtime")
+    assert built.returncode == 0, built.stderr[-2000:]
+    # a compiled-model file of the same forest, written by the library's own writer (through the host-side driver)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0:allocator_may_return_null=0:max_allocation_size_mb=4096",
+               TMPDIR=str(tmp_path))
+    run = subprocess.run([host_driver, json_path], capture_output=True, text=True, env=env, timeout=600)
+    assert run.returncode == 0, (run.stdout + run.stderr)[-3000:]
+    compiled = str(tmp_path / "sanitize_model.tbamd")
+    assert os.path.exists(compiled)
+    run = subprocess.run([exe, "600", "json", json_path, "onnx", onnx_path, "6", "compiled", compiled],
+                         capture_output=True, text=True, env=env, timeout=900)
+    assert run.returncode == 0, (run.stdout + run.stderr)[-4000:]
+    assert run.stdout.strip().endswith("ok"), run.stdout[-500:]
+
+
+@pytest.fixture(scope="module")
+def address_driver(tmp_path_factory):
+    """The runner driver under ASan + UBSan, built once for the tests that use it."""
+    return _build_runner_driver(tmp_path_factory.mktemp("address_driver"), "address,undefined")
+
+
+@pytest.fixture(scope="module")
+def host_driver(tmp_path_factory):
+    """tests/native/sanitize_host.cpp under ASan + UBSan, built once."""
+    where = tmp_path_factory.mktemp("host_driver")
+    exe = str(where / "sanitize_host")
+    flags = ["-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
+             "-fno-omit-frame-pointer", "-I", CSRC]
+    built = _compile_and_link(where, flags, [os.path.join(HERE, "native", "sanitize_host.cpp")] + [os.path.join(CSRC, s) for s in HOST_SOURCES], exe)
+    if built.returncode != 0 and "sanitize" in built.stderr:
+        pytest.skip("this g++ has no sanitizer runtime")
+    assert built.returncode == 0, built.stderr[-2000:]
+    return exe
+
+
 def _wide_model(tmp_path):
     """40 trees over 600 features: 8300 rows are 20 MB of input, enough for the host entry point to send them
     in pieces through its pinned buffers, and cheap to walk on the CPU."""
@@ -83,14 +133,41 @@ def _wide_model(tmp_path):
     return path
 
 
+def _multiclass_model(tmp_path):
+    """160 complete trees of depth 6 voting for 8 classes over 54 features: the shape of the multiclass benchmark
+    configuration at a fifth of its trees (every plan shape is re-packed under the sanitizers dozens of times)."""
+    import numpy as np
+    rng = np.random.Generator(np.random.PCG64(6))
+    trees = [synth._grow_tree(rng, 6, lambda d, s: 1.0, lambda: (rng.integers(0, 54), float(np.round(rng.normal(), 2))),
+                              lambda: rng.normal(0.0, 0.1)) for _ in range(160)]
+    path = str(tmp_path / "multiclass160.json")
+    synth.write_xgboost_json(path, trees, 54, objective="multi:softmax", num_class=8, tree_info=[t % 8 for t in range(160)])
+    return path
+
+
 @pytest.mark.skipif(shutil.which("g++") is None, reason="needs g++")
-def test_runner_under_address_sanitizer(tmp_path, synth_model):
-    exe = _build_runner_driver(tmp_path, "address,undefined")
-    args = [_wide_model(tmp_path), "8300", synth_model(4), "300", synth_model(3), "300", synth_model(1), "9000"]
+def test_runner_under_address_sanitizer(tmp_path, synth_model, address_driver):
+    exe = address_driver
+    args = [_wide_model(tmp_path), "8300", synth_model(4), "300", _multiclass_model(tmp_path), "300", synth_model(1), "9000"]
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", TMPDIR=str(tmp_path))
     run = subprocess.run([exe] + args, capture_output=True, text=True, env=env, timeout=900)
     assert run.returncode == 0, (run.stdout + run.stderr)[-4000:]
     assert run.stdout.strip().endswith("ok")
+
+
+@pytest.mark.skipif(shutil.which("g++") is None, reason="needs g++")
+def test_runner_survives_mutated_compiled_models(tmp_path, synth_model, address_driver):
+    """tbmi_load_compiled_model on compiled-model files whose header words (plan, batch size, return type, counts) and
+    body were overwritten: refused with a message or loaded and run on a few rows, under ASan + UBSan."""
+    exe = address_driver
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0:max_allocation_size_mb=8192", TMPDIR=str(tmp_path))
+    run = subprocess.run([exe, synth_model(1), "64"], capture_output=True, text=True, env=env, timeout=900)
+    assert run.returncode == 0, (run.stdout + run.stderr)[-4000:]
+    compiled = str(tmp_path / "sanitize_runner.tbamd")
+    assert os.path.exists(compiled)
+    run = subprocess.run([exe, "--mutate", compiled, "1500"], capture_output=True, text=True, env=env, timeout=900)
+    assert run.returncode == 0, (run.stdout + run.stderr)[-4000:]
+    assert run.stdout.strip().endswith("ok"), run.stdout[-500:]
 
 
 @pytest.mark.skipif(shutil.which("g++") is None, reason="needs g++")

@@ -46,7 +46,7 @@ struct Reader {
     const uint64_t n = Get<uint64_t>();
     if (n > (bytes.size() - pos) / sizeof(T)) throw Error("model file is truncated");
     std::vector<T> v(n);
-    std::memcpy(v.data(), bytes.data() + pos, n * sizeof(T));
+    if (n) std::memcpy(v.data(), bytes.data() + pos, n * sizeof(T));
     pos += n * sizeof(T);
     return v;
   }
@@ -128,7 +128,7 @@ CompiledModel LoadCompiledModel(const std::string &path) {
   m.plan.peelWalks = r.Get<int32_t>() != 0;
   m.plan.deferTails = r.Get<int32_t>() != 0;
   const uint64_t trees = r.Get<uint64_t>();
-  if (trees > bytes.size()) throw Error("model file is truncated");
+  if (trees > (bytes.size() - r.pos) / 36) throw Error("model file is truncated"); // (a tree takes 36 bytes at least)
   m.forest.trees.resize(trees);
   for (Tree &t : m.forest.trees) {
     t.classId = r.Get<int32_t>();

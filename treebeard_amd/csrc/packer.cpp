@@ -423,6 +423,15 @@ PackedModel PackForGlobalWalk(const Forest &forest, const LaunchPlan &plan) {
 } // namespace
 
 PackedModel PackForest(const Forest &input, const LaunchPlan &plan, const HitCountProfile *profile) {
+  // Plans also come out of files: every field is brought into its range before anything is computed from it.
+  if (plan.kernel != LaunchPlan::Kernel::kRowParallelLds && plan.kernel != LaunchPlan::Kernel::kTreeParallel &&
+      plan.kernel != LaunchPlan::Kernel::kGlobalWalk)
+    throw Error("launch plan names no kernel");
+  if (plan.rowsPerBlock < 1 || plan.rowsPerBlock > 1024 || plan.treeThreads < 1 || plan.treeThreads > 1024 || plan.treeLanes < 1 ||
+      plan.treeLanes > 1024)
+    throw Error("launch plan: rows per block, tree threads and tree lanes must be in [1, 1024]");
+  if (plan.treeSlices < 1 || plan.treeSlices > 65535) throw Error("launch plan: tree slices must be in [1, 65535]");
+  if (plan.tiling < 0 || plan.tiling > 2) throw Error("launch plan: tiling type must be 0, 1 or 2");
   const Forest forest = NormalizeToLessThan(input);
   if (profile && profile->hits.size() != forest.trees.size()) throw Error("hit-count profile does not match the forest");
   if (plan.kernel == LaunchPlan::Kernel::kGlobalWalk) {
