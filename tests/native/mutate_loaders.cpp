@@ -2,7 +2,7 @@
 // overwritten words, cut and doubled pieces.  A loader may refuse a file (tbamd::Error) or load it; a loaded forest
 // must pass Validate() or be refused there, and a validated forest must pack and unpack.  Anything else - a
 // sanitizer report, another exception type, an allocation sized by a corrupt count - fails the run.
-// usage: mutate_loaders <iterations> (<kind> <file> [<features>])...   kind: json | onnx | compiled
+// usage: mutate_loaders <iterations> (<kind> <file> [<features> | <model.json>])...   kind: json | onnx <features> | compiled | profile <model.json>
 #include "forest.h"
 #include "model_file.h"
 #include "packer.h"
@@ -77,6 +77,8 @@ int main(int argc, char **argv) {
     int features = 0;
     a += 2;
     if (kind == "onnx") features = std::atoi(argv[a++]);
+    Forest profiled; // kind "profile": the forest the hit-count profile belongs to
+    if (kind == "profile") profiled = LoadXGBoostJSON(argv[a++]);
     std::ifstream in(path, std::ios::binary);
     const std::vector<char> good((std::istreambuf_iterator<char>(in)), std::istreambuf_iterator<char>());
     if (good.empty()) { std::printf("cannot read %s\n", path.c_str()); return 65; }
@@ -88,6 +90,14 @@ int main(int argc, char **argv) {
       }
       try {
         Forest forest;
+        if (kind == "profile") {
+          const HitCountProfile profile = LoadHitCountProfile(profiled, scratch);
+          LaunchPlan plan = ChoosePlan(profiled, 4096, nullptr, limits);
+          plan.tileSize = 4, plan.tiling = 1, plan.peelWalks = true, plan.interleave = 2, plan.featureOffsetInWords = false;
+          (void)PackForest(profiled, plan, &profile); // tile membership and peel depths come out of the counts
+          ++loaded, ++packed;
+          continue;
+        }
         if (kind == "json") forest = LoadXGBoostJSON(scratch);
         else if (kind == "onnx") forest = LoadONNX(scratch, features);
         else {

@@ -95,7 +95,14 @@ def test_loaders_survive_mutated_files(tmp_path, host_driver):
     assert run.returncode == 0, (run.stdout + run.stderr)[-3000:]
     compiled = str(tmp_path / "sanitize_model.tbamd")
     assert os.path.exists(compiled)
-    run = subprocess.run([exe, "600", "json", json_path, "onnx", onnx_path, "6", "compiled", compiled],
+    # a hit-count profile of the same forest in the reference's format (src/utils/StatsUtils.cpp:10-52)
+    profile_path = str(tmp_path / "profile.csv")
+    with open(profile_path, "w") as fh:
+        fh.write("%d, 1000\n" % len(trees))
+        for t in trees:
+            leaves = [n for n in range(len(t.left)) if t.left[n] == -1]
+            fh.write(", ".join("%d, 0" % rng.integers(0, 1000) for _ in leaves) + "\n")
+    run = subprocess.run([exe, "600", "json", json_path, "onnx", onnx_path, "6", "compiled", compiled, "profile", profile_path, json_path],
                          capture_output=True, text=True, env=env, timeout=900)
     assert run.returncode == 0, (run.stdout + run.stderr)[-4000:]
     assert run.stdout.strip().endswith("ok"), run.stdout[-500:]
