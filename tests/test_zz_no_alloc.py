@@ -84,3 +84,41 @@ def test_no_alloc_entry_point_rejects_what_does_not_fit(synth_model):
     want = torch.zeros((rows - 1,), dtype=torch.int8, device="cuda")
     runner.run_device(dx.data_ptr(), want.data_ptr(), rows - 1)
     np.testing.assert_array_equal(out[:rows - 1].cpu().numpy(), want.cpu().numpy())
+
+
+@pytest.mark.parametrize("k,plan,rows", [(2, ("plan", 256, 4, 4, 16384, 6), 5000), (3, None, 9000), (3, ("plan", 256, 4, 4, 0, 2), 3000),
+                                         (4, None, 2000)])
+def test_no_alloc_entry_point_under_graph_capture(synth_model, k, plan, rows):
+    """What the entry point is for: recorded into a HIP graph (no allocation, no synchronisation, no memset on its
+    path) and replayed several times on new input, with eager work and synchronisations between the replays; every
+    replay gives what an eager call gives, and what the oracle gives."""
+    runner = _runner(synth_model(k), rows, k == 3)
+    if plan:
+        runner.set_plan(*plan[1:])
+    forest = model_io.load_xgboost_json(synth_model(k))
+    dtype = torch.int8 if runner.result_dtype() == np.int8 else torch.float32
+    fixed_in = torch.zeros((rows, forest.num_features), dtype=torch.float32, device="cuda")
+    fixed_out = torch.zeros((rows,), dtype=dtype, device="cuda")
+    eager = torch.zeros_like(fixed_out)
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):       # an eager call first: kernel attributes are set at a kernel's first launch
+        runner.run_device_noalloc(fixed_in.data_ptr(), fixed_out.data_ptr(), rows, side.cuda_stream)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        runner.run_device_noalloc(fixed_in.data_ptr(), fixed_out.data_ptr(), rows, torch.cuda.current_stream().cuda_stream)
+    for replay in range(3):
+        x = synth.CONFIGS[k].batch_rows(rows, seed_offset=30 + replay)
+        fixed_in.copy_(torch.from_numpy(x))
+        fixed_out.fill_(77)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        runner.run_device(fixed_in.data_ptr(), eager.data_ptr(), rows)
+        np.testing.assert_array_equal(fixed_out.cpu().numpy(), eager.cpu().numpy())
+        pred, _ = cpu_oracle.predict(forest, x)
+        if k == 3:
+            np.testing.assert_array_equal(fixed_out.cpu().numpy().astype(np.float32), pred.astype(np.float32))
+        else:
+            np.testing.assert_allclose(fixed_out.cpu().numpy(), pred, rtol=1e-5, atol=1e-6)
