@@ -8,6 +8,7 @@
 // result initialisation and sigmoid).
 #include "kernels.h"
 
+#include <atomic>
 #include <cmath>
 
 namespace tbamd {
@@ -1288,13 +1289,13 @@ __global__ void __launch_bounds__(256) FinalizeWideKernel(const FinalizeParams p
 // time).  Two threads that meet here for the first time both make the call, which is harmless.
 template <auto Kernel> hipError_t AllowFullLds() {
   constexpr int kMaxDevices = 64;
-  static signed char raised[kMaxDevices] = {};
+  static std::atomic<bool> raised[kMaxDevices];
   int device = 0;
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess) return e;
-  if (device >= 0 && device < kMaxDevices && raised[device]) return hipSuccess;
+  if (device >= 0 && device < kMaxDevices && raised[device].load(std::memory_order_acquire)) return hipSuccess;
   e = hipFuncSetAttribute(reinterpret_cast<const void *>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-  if (e == hipSuccess && device >= 0 && device < kMaxDevices) raised[device] = 1;
+  if (e == hipSuccess && device >= 0 && device < kMaxDevices) raised[device].store(true, std::memory_order_release);
   return e;
 }
 
